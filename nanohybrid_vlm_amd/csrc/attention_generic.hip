@@ -7,6 +7,9 @@
 // start of the request), else 0. Value heads may have another size (E) than key heads (D).
 // Keys are taken in blocks of 64 aligned to absolute positions, always in rising
 // order, so the result for a position does not depend on the batch or the portion.
+// Options that a layer may name: a cap on the scores (s <- cap tanh(s / cap), after the scale), one more term in the
+// softmax's denominator (a sink: a key of a given score that has no value), and a gate per (token, head) whose
+// sigmoid multiplies the head's result (read from rows ``gate_ld`` entries apart).
 // This is the attention of the 32-bit path and the fallback of the bfloat16 path.
 #include "nhv_common.h"
 #include <math.h>
@@ -17,7 +20,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     const int* __restrict__ token_req, const int* __restrict__ positions, const int* __restrict__ block_tables,
-    int max_blocks, int n_items, int Hq, int Hkv, int D, int E, int page_size, float scale, int window, int chunk) {
+    int max_blocks, int n_items, int Hq, int Hkv, int D, int E, int page_size, float scale, int window, int chunk,
+    float cap, int has_sink, float sink, const T* __restrict__ gate, long long gate_ld) {
   extern __shared__ float q_s[];            // 4 waves x D floats
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave;
@@ -53,6 +57,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32(kr[d]), dot);
       s = dot * scale;
+      if (cap > 0.f) s = cap * tanhf(s / cap);
     }
     const float m_new = fmaxf(m, wave_max(s));     // finite: every block holds at least one visible key
     const float alpha = expf(m - m_new);           // 0 on the first block
@@ -74,7 +79,15 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
       }
     }
   }
-  const float inv = 1.0f / l;
+  if (has_sink) {                                  // the sink joins the denominator as one more key would, without a value
+    const float m_new = fmaxf(m, sink);
+    const float alpha = expf(m - m_new);
+    l = l * alpha + expf(sink - m_new);
+#pragma unroll
+    for (int i = 0; i < MAX_D_CHUNKS; ++i) acc[i] *= alpha;
+  }
+  float inv = 1.0f / l;
+  if (gate) inv /= 1.0f + expf(-to_f32(gate[(size_t)t * gate_ld + h]));
   T* o = out + ((size_t)t * Hq + h) * E;
 #pragma unroll
   for (int i = 0; i < MAX_D_CHUNKS; ++i) {
@@ -86,7 +99,9 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
 extern "C" int nhv_paged_attention_generic(const void* q, const void* k_cache, const void* v_cache, void* out,
                                            const void* token_req, const void* positions, const void* block_tables,
                                            int max_blocks, int T, int Hq, int Hkv, int D, int E, int page_size,
-                                           float scale, int window, int chunk, int dtype, void* stream) {
+                                           float scale, int window, int chunk, float cap, int has_sink, float sink,
+                                           const void* gate, long long gate_ld, int dtype, void* stream) {
+  NHV_REQUIRE(cap >= 0.f && (!gate || gate_ld >= Hq), "attention: cap %g, gate rows %lld apart for %d heads", (double)cap, gate_ld, Hq);
   NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && D > 0 && page_size > 0 && max_blocks > 0,
               "attention: bad sizes T=%d Hq=%d Hkv=%d D=%d page=%d blocks=%d", T, Hq, Hkv, D, page_size, max_blocks);
   NHV_REQUIRE(Hq % Hkv == 0, "attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
@@ -102,12 +117,12 @@ extern "C" int nhv_paged_attention_generic(const void* q, const void* k_cache, c
     hipLaunchKernelGGL(paged_attention_generic_kernel<float>, dim3(blocks), dim3(256), lds, s, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, (float*)out, (const int*)token_req,
                        (const int*)positions, (const int*)block_tables, max_blocks, (int)n_items, Hq, Hkv, D, E, page_size,
-                       scale, window, chunk);
+                       scale, window, chunk, cap, has_sink, sink, (const float*)gate, gate_ld);
   else if (dtype == NHV_BF16)
     hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, dim3(blocks), dim3(256), lds, s, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, (const int*)token_req,
                        (const int*)positions, (const int*)block_tables, max_blocks, (int)n_items, Hq, Hkv, D, E, page_size,
-                       scale, window, chunk);
+                       scale, window, chunk, cap, has_sink, sink, (const bf16_t*)gate, gate_ld);
   else
     return nhv_fail("attention: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("paged_attention_generic");

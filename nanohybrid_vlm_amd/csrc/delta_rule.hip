@@ -1,13 +1,15 @@
 // The gated delta rule: a recurrent mixer whose state is one matrix S[D, E] per head and request,
 //   S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t,
-// with a decay g_t per key channel, preceded by short causal convolutions over time on q, k and v.
+// with a decay g_t per key channel (or one per head: ``Dd`` = 1 below), preceded by short causal convolutions over time
+// on q, k and v.
 // Four kernels, the same for prompt portions and for single decoded tokens:
 //  - nhv_delta_prepare: per token, the convolutions (earlier inputs come from the step's own rows or from the
 //    request's kept inputs), SiLU, unit length per head for q and k, the decays from their linear part, beta;
 //  - nhv_conv_state_update: per request, the last taps - 1 inputs are kept for the next step;
 //  - nhv_delta_rule: per (request, head, tile of value columns), the recurrence over the step's tokens in order,
 //    from the request's state (zero for a request that starts at position 0) and back into it;
-//  - nhv_gated_head_norm: per (token, head), o over its root mean square, times a weight, times sigmoid(gate).
+//  - nhv_gated_head_norm: per (token, head), o over its root mean square, times a weight, times sigmoid(gate) or
+//    gate sigmoid(gate).
 // Everything here is float: the state, the decays, the unit vectors, the sums. A column of S (one value channel)
 // never meets another column, so a block owns a tile of columns, a column belongs to R adjacent lanes that hold D / R
 // entries each, and the two sums over D per token are taken with lane shuffles; the tokens' vectors come through
@@ -24,16 +26,18 @@ __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log
 // ---------------------------------------------------------------- per token: what enters the recurrence
 // proj[T, ld]: q (G D) | k (G D) | v (H E) | beta (H) as the projection left them. taps[C, n], C = 2 G D + H E, last
 // column for the token itself. kept[slots, C, n - 1]: the inputs at the n - 1 positions before the request's first
-// token of this step. a_lin[T, H D]: the decays' linear part on entry, the decays on return.
+// token of this step. a_lin: the decays' linear part, rows of H Dd floats ``a_ld`` apart (a tensor of its own, or
+// columns of a float projection); decay_out[T, H Dd]: the decays (it may be a_lin itself where that is dense); Dd = D
+// (a decay per key channel) or 1 (one per head); dt_bias[H Dd].
 // One wave per (token, unit); the units of a token are its 2 G query and key heads (D channels each), its H value
 // heads (E channels), its H heads of decays (D channels) and its H betas (one unit).
 template <typename TI>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const TI* __restrict__ proj, int ld, const float* __restrict__ taps, int n_taps, const float* __restrict__ kept,
-    float* __restrict__ a_lin, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+    const float* a_lin, long long a_ld, float* decay_out, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
     const int* __restrict__ token_req, const int* __restrict__ positions, const int* __restrict__ cu,
     const int* __restrict__ state_slots, float* __restrict__ q_out, float* __restrict__ k_out, float* __restrict__ v_out,
-    float* __restrict__ beta_out, int H, int G, int D, int E) {
+    float* __restrict__ beta_out, int H, int G, int D, int E, int Dd) {
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int unit = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -47,9 +51,8 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
   if (unit >= 2 * G + H) {
     const int h = unit - 2 * G - H;
     const float rate = expf(a_log[h]);
-    for (int d = lane; d < D; d += NHV_WAVE) {
-      const size_t at = (size_t)t * H * D + h * D + d;
-      a_lin[at] = expf(-rate * softplus_f(a_lin[at] + dt_bias[h * D + d]));
+    for (int d = lane; d < Dd; d += NHV_WAVE) {
+      decay_out[(size_t)t * H * Dd + h * Dd + d] = expf(-rate * softplus_f(a_lin[(size_t)t * a_ld + h * Dd + d] + dt_bias[h * Dd + d]));
     }
     return;
   }
@@ -93,21 +96,26 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
   }
 }
 
-extern "C" int nhv_delta_prepare(const void* proj, int proj_dtype, const void* taps, int n_taps, const void* kept,
-                                 void* a_lin, const void* dt_bias, const void* a_log, const void* token_req,
+extern "C" int nhv_delta_prepare(const void* proj, int proj_dtype, int ld, const void* taps, int n_taps, const void* kept,
+                                 const void* a_lin, long long a_ld, void* decay_out, const void* dt_bias, const void* a_log, const void* token_req,
                                  const void* positions, const void* cu, const void* state_slots, void* q_out, void* k_out,
-                                 void* v_out, void* beta_out, int T, int H, int G, int D, int E, void* stream) {
+                                 void* v_out, void* beta_out, int T, int H, int G, int D, int E, int decay_dim, void* stream) {
   NHV_REQUIRE(T > 0 && H > 0 && G > 0 && D > 0 && E > 0 && H % G == 0, "delta_prepare: bad sizes T=%d H=%d G=%d D=%d E=%d", T, H, G, D, E);
+  NHV_REQUIRE(decay_dim == D || decay_dim == 1, "delta_prepare: %d decays a head (one, or one per key channel: %d)", decay_dim, D);
   NHV_REQUIRE(n_taps >= 1 && n_taps <= NHV_MAX_TAPS, "delta_prepare: %d taps (1 to %d are taken)", n_taps, NHV_MAX_TAPS);
   NHV_REQUIRE(D <= 1024 && E <= 1024 && 2 * G + 2 * H + 1 <= 4 * 65535, "delta_prepare: D=%d, E=%d (up to 1024 each), %d heads", D, E, H);
   const int C = 2 * G * D + H * E;
+  NHV_REQUIRE(ld >= C + H && a_ld >= (long long)H * decay_dim, "delta_prepare: rows of %d entries for %d, decays' rows of %lld for %d", ld, C + H,
+              a_ld, H * decay_dim);
   const int n_units = 2 * G + 2 * H + 1;
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(TI)                                                                                                    \
-  hipLaunchKernelGGL(delta_prepare_kernel<TI>, dim3(T, (n_units + 3) / 4), dim3(256), 0, s, (const TI*)proj, C + H,   \
-                     (const float*)taps, n_taps, (const float*)kept, (float*)a_lin, (const float*)dt_bias,            \
+  hipLaunchKernelGGL(delta_prepare_kernel<TI>, dim3(T, (n_units + 3) / 4), dim3(256), 0, s, (const TI*)proj, ld,      \
+                     (const float*)taps, n_taps, (const float*)kept, (const float*)a_lin, a_ld, (float*)decay_out,    \
+                     (const float*)dt_bias,                                                                           \
                      (const float*)a_log, (const int*)token_req, (const int*)positions, (const int*)cu,               \
-                     (const int*)state_slots, (float*)q_out, (float*)k_out, (float*)v_out, (float*)beta_out, H, G, D, E)
+                     (const int*)state_slots, (float*)q_out, (float*)k_out, (float*)v_out, (float*)beta_out, H, G, D, E,  \
+                     decay_dim)
   if (proj_dtype == NHV_F32) LAUNCH(float);
   else if (proj_dtype == NHV_BF16) LAUNCH(bf16_t);
   else return nhv_fail("delta_prepare: unknown dtype %d", proj_dtype);
@@ -187,7 +195,7 @@ template <int DR, int R, bool DIRECT>
 __global__ __launch_bounds__(256) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ decay,
     const float* __restrict__ beta, float* __restrict__ state, float* __restrict__ out, const int* __restrict__ positions,
-    const int* __restrict__ cu, const int* __restrict__ state_slots, int H, int G, int D, int E, int cols, int tile) {
+    const int* __restrict__ cu, const int* __restrict__ state_slots, int H, int G, int D, int E, int cols, int tile, int Dd) {
   extern __shared__ __attribute__((aligned(16))) float staged[];   // 2 buffers of tile * row floats, row = 3 Dp + cols + 1 (rounded up to 4), Dp = R DR
   const int req = blockIdx.z, h = blockIdx.y;
   const int first = cu[req], end = cu[req + 1];
@@ -224,15 +232,17 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     for (int t = first; t < end; ++t) {
       const float* qr = q + ((size_t)t * G + g) * D;
       const float* kr = k + ((size_t)t * G + g) * D;
-      const float* gr = decay + ((size_t)t * H + h) * D;
+      const float* gr = decay + ((size_t)t * H + h) * Dd;
+      const bool one_decay = Dd == 1;      // (one number a head: every key channel decays alike)
       float cq[DR], ck[DR];
       float k_s = 0.f, q_s = 0.f, q_k = 0.f;
 #pragma unroll
       for (int i = 0; i < DR; i += 4) {
         float qv[4], kv[4], gv[4];
         if (whole4 && d0 + i < D) {
-          const float4 q4 = *reinterpret_cast<const float4*>(qr + d0 + i), k4 = *reinterpret_cast<const float4*>(kr + d0 + i),
-                       g4 = *reinterpret_cast<const float4*>(gr + d0 + i);
+          const float4 q4 = *reinterpret_cast<const float4*>(qr + d0 + i), k4 = *reinterpret_cast<const float4*>(kr + d0 + i);
+          const float g1 = one_decay ? gr[0] : 0.f;
+          const float4 g4 = one_decay ? float4{g1, g1, g1, g1} : *reinterpret_cast<const float4*>(gr + d0 + i);
           qv[0] = q4.x; qv[1] = q4.y; qv[2] = q4.z; qv[3] = q4.w;
           kv[0] = k4.x; kv[1] = k4.y; kv[2] = k4.z; kv[3] = k4.w;
           gv[0] = g4.x; gv[1] = g4.y; gv[2] = g4.z; gv[3] = g4.w;
@@ -242,7 +252,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
             const bool ok = !whole4 && d0 + i + j < D;
             qv[j] = ok ? qr[d0 + i + j] : 0.f;
             kv[j] = ok ? kr[d0 + i + j] : 0.f;
-            gv[j] = ok ? gr[d0 + i + j] : 0.f;
+            gv[j] = ok ? gr[one_decay ? 0 : d0 + i + j] : 0.f;
           }
         }
 #pragma unroll
@@ -283,8 +293,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
         const int which = c / Dp, d = c % Dp;
         if (d < D) {
           src[j] = which == 0 ? q + ((size_t)tt * G + g) * D + d : which == 1 ? k + ((size_t)tt * G + g) * D + d
-                                                                              : decay + ((size_t)tt * H + h) * D + d;
-          stride[j] = which == 2 ? H * D : G * D;
+                                                                              : decay + ((size_t)tt * H + h) * Dd + (Dd == 1 ? 0 : d);
+          stride[j] = which == 2 ? H * Dd : G * D;
         }
       } else if (c < 3 * Dp + cols) {
         const int ee = e0 + c - 3 * Dp;
@@ -383,8 +393,9 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
 
 extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const void* decay, const void* beta, void* state,
                               void* out, const void* positions, const void* cu, const void* state_slots, int B, int H, int G,
-                              int D, int E, int max_q_len, void* stream) {
+                              int D, int E, int max_q_len, int decay_dim, void* stream) {
   NHV_REQUIRE(B > 0 && H > 0 && G > 0 && D > 0 && E > 0 && H % G == 0, "delta_rule: bad sizes B=%d H=%d G=%d D=%d E=%d", B, H, G, D, E);
+  NHV_REQUIRE(decay_dim == D || decay_dim == 1, "delta_rule: %d decays a head (one, or one per key channel: %d)", decay_dim, D);
   NHV_REQUIRE(D <= 1024 && B <= 65535 && H <= 65535, "delta_rule: D=%d (up to 1024), B=%d, H=%d (up to 65535)", D, B, H);
   // entries a lane: 4, or what keeps a column within the 64 lanes of a wave. (A token's time is what a wave has to
   // issue for it, not its arithmetic: 2,048 tokens of 16 heads of 128 x 128 took 890 us with 8 entries a lane and 700 us
@@ -413,7 +424,7 @@ extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const
 #define LAUNCH_AS(DRV, RV, DIR)                                                                                       \
   hipLaunchKernelGGL((delta_rule_kernel<DRV, RV, DIR>), grid, block, lds, s, (const float*)q, (const float*)k,        \
                      (const float*)v, (const float*)decay, (const float*)beta, (float*)state, (float*)out,            \
-                     (const int*)positions, (const int*)cu, (const int*)state_slots, H, G, D, E, cols, tile)
+                     (const int*)positions, (const int*)cu, (const int*)state_slots, H, G, D, E, cols, tile, decay_dim)
 #define LAUNCH(DRV, RV)               \
   do {                                \
     if (direct) LAUNCH_AS(DRV, RV, true); \
@@ -438,10 +449,12 @@ extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const
 }
 
 // ---------------------------------------------------------------- the read-out's norm and gate
-// y[t, h, e] = o[t, h, e] / sqrt(mean over e of o^2 + eps) * w[e] * sigmoid(gate[t, h, e]); one wave per (t, h).
+// y[t, h, e] = o[t, h, e] / sqrt(mean over e of o^2 + eps) * w[e] * f(gate[t, h, e]) (the gates' rows ``gate_ld`` floats apart), f the sigmoid (gate_act 0) or
+// z sigmoid(z) (1); one wave per (t, h).
 template <typename TO>
-__global__ void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ gate, const float* __restrict__ w,
-                                       TO* __restrict__ y, int E, float eps, int n_items) {
+__global__ void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ gate, long long gate_ld, int H,
+                                       const float* __restrict__ w,
+                                       TO* __restrict__ y, int E, float eps, int n_items, int gate_act) {
   const int item = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (item >= n_items) return;
   const int lane = threadIdx.x & 63;
@@ -450,21 +463,26 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float*
   for (int e = lane; e < E; e += NHV_WAVE) ss = fmaf(src[e], src[e], ss);
   const float r = 1.0f / sqrtf(wave_sum(ss) / (float)E + eps);
   for (int e = lane; e < E; e += NHV_WAVE)
-    y[(size_t)item * E + e] = from_f32<TO>(src[e] * r * w[e] * sigmoid_f(gate[(size_t)item * E + e]));
+  {
+    const float z = gate[(size_t)(item / H) * gate_ld + (size_t)(item % H) * E + e];
+    y[(size_t)item * E + e] = from_f32<TO>(src[e] * r * w[e] * (gate_act == 1 ? silu_f(z) : sigmoid_f(z)));
+  }
 }
 
-extern "C" int nhv_gated_head_norm(const void* o, const void* gate, const void* w, void* y, int T, int H, int E, float eps,
-                                   int y_dtype, void* stream) {
+extern "C" int nhv_gated_head_norm(const void* o, const void* gate, long long gate_ld, const void* w, void* y, int T, int H, int E, float eps,
+                                   int y_dtype, int gate_act, void* stream) {
+  NHV_REQUIRE(gate_ld >= (long long)H * E, "gated_head_norm: gate rows %lld apart for %d entries", gate_ld, H * E);
+  NHV_REQUIRE(gate_act == 0 || gate_act == 1, "gated_head_norm: gate activation %d (0: sigmoid, 1: SiLU)", gate_act);
   NHV_REQUIRE(T > 0 && H > 0 && E > 0 && (long long)T * H < (1ll << 31), "gated_head_norm: bad sizes T=%d H=%d E=%d", T, H, E);
   const int n_items = T * H;
   const unsigned blocks = (unsigned)((n_items + 3) / 4);
   hipStream_t s = (hipStream_t)stream;
   if (y_dtype == NHV_F32)
     hipLaunchKernelGGL(gated_head_norm_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)o, (const float*)gate,
-                       (const float*)w, (float*)y, E, eps, n_items);
+                       gate_ld, H, (const float*)w, (float*)y, E, eps, n_items, gate_act);
   else if (y_dtype == NHV_BF16)
     hipLaunchKernelGGL(gated_head_norm_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const float*)o, (const float*)gate,
-                       (const float*)w, (bf16_t*)y, E, eps, n_items);
+                       gate_ld, H, (const float*)w, (bf16_t*)y, E, eps, n_items, gate_act);
   else return nhv_fail("gated_head_norm: unknown dtype %d", y_dtype);
   NHV_LAUNCH_CHECK("gated_head_norm");
   return 0;

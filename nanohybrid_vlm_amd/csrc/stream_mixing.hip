@@ -194,15 +194,16 @@ __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __
 
 extern "C" int nhv_rotary_split_write(const void* qkv, const void* bias, const void* qk_freqs, int rot, const void* v_freqs,
                                       const void* positions, const void* slot_mapping, void* q_out, void* k_cache,
-                                      void* v_cache, int T, int Hq, int Hkv, int D, int E, int with_kv, int dtype,
-                                      void* stream) {
+                                      void* v_cache, int T, int Hq, int Hkv, int D, int E, int with_kv, int more_columns,
+                                      int dtype, void* stream) {
+  NHV_REQUIRE(more_columns >= 0, "rotary_split_write: %d columns after the projection", more_columns);
   NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && D > 0 && E > 0, "rotary_split_write: bad sizes T=%d Hq=%d Hkv=%d D=%d E=%d", T, Hq, Hkv, D, E);
   NHV_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "rotary_split_write: rotary size %d with head size %d", rot, D);
   NHV_REQUIRE(rot == 0 || qk_freqs, "rotary_split_write: a rotary size without frequencies");
   NHV_REQUIRE(!v_freqs || E % 2 == 0, "rotary_split_write: value heads of odd size %d cannot be turned", E);
   NHV_REQUIRE(!with_kv || (slot_mapping && k_cache && v_cache), "rotary_split_write: cache write without cache");
   const int heads = with_kv ? Hq + 2 * Hkv : Hq;
-  const int ld = with_kv ? Hq * D + Hkv * (D + E) : Hq * D;
+  const int ld = (with_kv ? Hq * D + Hkv * (D + E) : Hq * D) + more_columns;   // (columns that belong to another reader)
   NHV_REQUIRE((long long)T * heads < (1ll << 31), "rotary_split_write: too many tokens");
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(TT)                                                                                                   \

@@ -20,7 +20,7 @@ from . import library
 
 CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "gemm_fewrows_bf16.hip", "attention_generic.hip",
                 "sampling.hip", "measure.hip", "stream_mixing.hip", "delta_rule.hip", "parallel_block.hip", "latent_attention.hip",
-                "routed_experts.hip"]
+                "routed_experts.hip", "hyper_streams.hip"]
 BLAS_SOURCES = ["error.hip", "gemm_library.hip"]                                                   # the vendor's matrix library, algorithm by number
 BLAS_LINK = ["-lhipblaslt"]
 ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefill_bf16.hip"]      # compiled once per head size
@@ -91,6 +91,14 @@ class AttentionBatch:
     context_lens: torch.Tensor     # [B] keys of the request after this step
     max_q_len: int
     max_context_len: int
+
+
+def _gate_args(gate):
+    """(pointer to the first gate of the first row, entries between rows) of a gate given as (tensor, first column)."""
+    if gate is None:
+        return ctypes.c_void_p(0), ctypes.c_longlong(0)
+    t, col = gate
+    return ctypes.c_void_p(t.data_ptr() + col * t.element_size()), ctypes.c_longlong(t.shape[1])
 
 
 class NativeBackend:
@@ -176,12 +184,17 @@ class NativeBackend:
                    _ptr(q_out), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], Hq, Hkv, D, int(write_kv),
                    dtype_code(qkv), wd, _stream())
 
-    def paged_attention(self, q, k_cache, v_cache, out, batch: AttentionBatch, block_tables, scale, window, chunk=0):
+    def paged_attention(self, q, k_cache, v_cache, out, batch: AttentionBatch, block_tables, scale, window, chunk=0,
+                        cap=0.0, sink=None, gate=None):
+        """``cap``: scores become cap tanh(score / cap); ``sink``: the score of one more term in the denominator;
+        ``gate`` = (tensor [tokens, columns] of q's element type, first column): the sigmoid of column + head
+        multiplies the head's result."""
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
         E = v_cache.shape[3]
+        plain = not cap and sink is None and gate is None
         # the kernels on the matrix cores take value heads of the key heads' size; a chunk goes to them as a negative window
-        fast = q.dtype == torch.bfloat16 and E == D and D % 16 == 0 and D <= 256
+        fast = plain and q.dtype == torch.bfloat16 and E == D and D % 16 == 0 and D <= 256
         if chunk:
             window = -chunk
         if fast and batch.max_q_len == 1 and Hq // Hkv <= 16 and T <= 65535:
@@ -201,7 +214,8 @@ class NativeBackend:
                               ctypes.c_float(scale), window, _stream(), lib=self.attention_lib(D))
         self._call("nhv_paged_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
                    _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables), block_tables.shape[1], T, Hq, Hkv,
-                   D, E, page_size, ctypes.c_float(scale), 0 if chunk else window, chunk, dtype_code(q), _stream())
+                   D, E, page_size, ctypes.c_float(scale), 0 if chunk else window, chunk, ctypes.c_float(cap or 0.0),
+                   int(sink is not None), ctypes.c_float(sink or 0.0), *_gate_args(gate), dtype_code(q), _stream())
 
     # -- layers that are not the pre-norm kind: norms with one number, sums over depth, rotation without a table --
     def scalar_rmsnorm(self, x, gain, y, eps):
@@ -222,20 +236,26 @@ class NativeBackend:
                    _ptr(wb), ctypes.c_float(pair_eps), dtype_code(a), _stream())
 
     def rotary_split_write(self, qkv, bias, qk_freqs, rot, v_freqs, positions, slot_mapping, q_out, k_cache, v_cache,
-                           Hq, Hkv, D, E, with_kv):
+                           Hq, Hkv, D, E, with_kv, more_columns=0):
         self._call("nhv_rotary_split_write", _ptr(qkv), _ptr(bias), _ptr(qk_freqs), rot, _ptr(v_freqs), _ptr(positions),
                    _ptr(slot_mapping), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], Hq, Hkv, D, E,
-                   int(with_kv), dtype_code(qkv), _stream())
+                   int(with_kv), more_columns, dtype_code(qkv), _stream())
 
     def turn_back(self, x, freqs, positions):
         T, H, E = x.shape
         self._call("nhv_turn_back", _ptr(x), _ptr(freqs), _ptr(positions), T, H, E, dtype_code(x), _stream())
 
     # -- the gated delta rule --
-    def delta_prepare(self, proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E):
-        self._call("nhv_delta_prepare", _ptr(proj), dtype_code(proj), _ptr(taps), taps.shape[1], _ptr(kept), _ptr(a_lin),
-                   _ptr(dt_bias), _ptr(a_log), _ptr(batch.token_req), _ptr(batch.positions), _ptr(batch.cu_seqlens_q),
-                   _ptr(state_slots), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), proj.shape[0], H, G, D, E, _stream())
+    def delta_prepare(self, proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E,
+                      decay=None, a_col=0):
+        """``a_lin`` [tokens, columns] float32: the decays' linear part from column ``a_col`` on; ``decay``
+        [tokens, heads, 1 or D]: where the decays go (None: into ``a_lin`` itself, which then holds nothing else)."""
+        decay_dim = D if decay is None else decay.shape[2]
+        self._call("nhv_delta_prepare", _ptr(proj), dtype_code(proj), proj.shape[1], _ptr(taps), taps.shape[1], _ptr(kept),
+                   ctypes.c_void_p(a_lin.data_ptr() + 4 * a_col), ctypes.c_longlong(a_lin.shape[1]),
+                   _ptr(a_lin if decay is None else decay), _ptr(dt_bias), _ptr(a_log), _ptr(batch.token_req),
+                   _ptr(batch.positions), _ptr(batch.cu_seqlens_q), _ptr(state_slots), _ptr(q), _ptr(k), _ptr(v), _ptr(beta),
+                   proj.shape[0], H, G, D, E, decay_dim, _stream())
 
     def conv_state_update(self, proj, kept, n_taps, batch, state_slots, channels):
         self._call("nhv_conv_state_update", _ptr(proj), dtype_code(proj), proj.shape[1], _ptr(kept), n_taps,
@@ -247,12 +267,36 @@ class NativeBackend:
         _, H, E = v.shape
         self._call("nhv_delta_rule", _ptr(q), _ptr(k), _ptr(v), _ptr(decay), _ptr(beta), _ptr(state), _ptr(out),
                    _ptr(batch.positions), _ptr(batch.cu_seqlens_q), _ptr(state_slots), batch.num_requests, H, G, D, E,
-                   max(1, batch.max_q_len), _stream())
+                   max(1, batch.max_q_len), decay.shape[2], _stream())
 
-    def gated_head_norm(self, o, gate, w, y, eps):
+    def gated_head_norm(self, o, gate, w, y, eps, gate_col=0, gate_act=0):
+        """``gate`` [tokens, columns] float32: the gates of (t, h, e) from column ``gate_col`` on; ``gate_act`` 0: the
+        sigmoid, 1: SiLU."""
         T, H, E = o.shape
-        self._call("nhv_gated_head_norm", _ptr(o), _ptr(gate), _ptr(w), _ptr(y), T, H, E, ctypes.c_float(eps),
-                   dtype_code(y), _stream())
+        self._call("nhv_gated_head_norm", _ptr(o), ctypes.c_void_p(gate.data_ptr() + 4 * gate_col),
+                   ctypes.c_longlong(gate.shape[1]), _ptr(w), _ptr(y), T, H, E, ctypes.c_float(eps), dtype_code(y),
+                   gate_act, _stream())
+
+    # -- several residual streams side by side, and what models on them need --
+    def streams_step(self, X, x0, mix, out_w, a, b, sa, sb, in_w, norm_w, eps, h, total, n, T, W, rows_dtype):
+        self._call("nhv_streams_step", _ptr(X), ctypes.c_longlong(0 if X is None else X.stride(0)), _ptr(x0), _ptr(mix),
+                   _ptr(out_w), _ptr(a), _ptr(b), ctypes.c_float(sa), ctypes.c_float(sb), _ptr(in_w), _ptr(norm_w),
+                   ctypes.c_float(eps), _ptr(h), _ptr(total), n, T, W, _DTYPE_CODE[rows_dtype], _stream())
+
+    def embed_float(self, ids, table, out, scale):
+        T, W = out.shape
+        self._call("nhv_embed_float", _ptr(ids), _ptr(table), _ptr(out), T, W, table.shape[0], dtype_code(table),
+                   ctypes.c_float(scale), _stream())
+
+    def activation(self, x, act):
+        self._call("nhv_activation", _ptr(x), ctypes.c_size_t(x.numel()), act, dtype_code(x), _stream())
+
+    def scaled_sum(self, a, b, y, sa, sb):
+        self._call("nhv_scaled_sum", _ptr(a), _ptr(b), _ptr(y), ctypes.c_size_t(y.numel()), ctypes.c_float(sa),
+                   ctypes.c_float(sb), dtype_code(a), _stream())
+
+    def scale(self, x, factor):
+        self._call("nhv_scale", _ptr(x), ctypes.c_size_t(x.numel()), ctypes.c_float(factor), _stream())
 
     # -- layers of two norms side by side, an embedding with a hashed pair row --
     def embed_pair_hash(self, ids, table, pair_table, out, batch, state_slots, prev_state, buckets, mul_prev, mul_cur):
@@ -858,7 +902,7 @@ def dense(x):
         return x.tensor()
     if isinstance(x, Summed):
         raise KernelError("a sum that was made for a norm (ops.Summed) goes through that norm, not anywhere else")
-    if isinstance(x, NormedPairMean):
+    if isinstance(x, (NormedPairMean, ScaledPairSum)):
         return x.tensor()
     return x
 
@@ -1009,10 +1053,14 @@ def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_m
 
 
 def paged_attention(q, k_cache, v_cache, batch: AttentionBatch, block_tables, scale: float,
-                    window: int | None = None, chunk: int | None = None) -> torch.Tensor:
+                    window: int | None = None, chunk: int | None = None, softcap: float | None = None,
+                    sink: float | None = None, gate: tuple | None = None) -> torch.Tensor:
     """Every query reads its request's keys up to its own position: all of them, the last ``window``, or (``chunk``)
     those of its own block of ``chunk`` positions counted from the request's start. The value heads may have another
-    size than the key heads: the result is [tokens, heads, value size]."""
+    size than the key heads: the result is [tokens, heads, value size].
+    ``softcap``: a score s (after the scale) becomes softcap tanh(s / softcap). ``sink``: the softmax's denominator
+    holds one more term exp(sink), a key of that score without a value. ``gate`` = (rows [tokens, columns] of q's
+    element type, first column): head h's result at token t is multiplied by sigmoid(rows[t, first column + h])."""
     _need(q.dim() == 3, "attention: q must be [tokens, heads, head_dim]")
     T, Hq, D = q.shape
     _dense(q, "attention: q")
@@ -1037,10 +1085,22 @@ def paged_attention(q, k_cache, v_cache, batch: AttentionBatch, block_tables, sc
           lambda: f"attention: block tables of {block_tables.shape[1]} pages of {page_size} are too short for "
           f"{batch.max_context_len} keys")
     out = torch.empty((T, Hq, v_cache.shape[3]), dtype=q.dtype, device=q.device)
+    more = {}
+    if softcap is not None:
+        _need(softcap > 0, lambda: f"attention: the cap on scores must be positive, got {softcap}")
+        more["cap"] = float(softcap)
+    if sink is not None:
+        more["sink"] = float(sink)
+    if gate is not None:
+        rows, col = gate
+        _need(rows.dim() == 2 and rows.shape[0] == T and 0 <= col and col + Hq <= rows.shape[1],
+              lambda: f"attention: gates {tuple(rows.shape)} for {Hq} heads from column {col}")
+        _dense(rows, "attention: gates", dtype=q.dtype)
+        more["gate"] = (rows, int(col))
     if chunk:
-        backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), 0, int(chunk))
+        backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), 0, int(chunk), **more)
     else:
-        backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), int(window or 0))
+        backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), int(window or 0), **more)
     return out
 
 
@@ -1128,7 +1188,8 @@ def gated_linear(x, w: torch.Tensor, activation: str = "silu") -> torch.Tensor:
 
 
 # ------------------------------------------------------------------ two norms side by side, a hashed pair embedding
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}            # what a gate may pass (``gated_linear``, ``act_mul``)
+PLAIN_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu2": 2}    # what rows may pass on their own (``activation_``); relu2: max(z, 0)^2
 
 
 def embed_pair_hash(ids: torch.Tensor, table: torch.Tensor, pair_table: torch.Tensor, batch: AttentionBatch,
@@ -1425,14 +1486,17 @@ def depth_mix(x: torch.Tensor, a, b: torch.Tensor | None, results: torch.Tensor,
 
 def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: torch.Tensor | None,
                        v_freqs: torch.Tensor | None, positions: torch.Tensor, slot_mapping, k_cache, v_cache,
-                       num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, with_kv: bool = True) -> torch.Tensor:
-    """Splits the packed projection q | k | v (``with_kv``) or q alone, adds the bias, turns pair (i, i + r) of every
+                       num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, with_kv: bool = True,
+                       more_columns: int = 0) -> torch.Tensor:
+    """Splits the packed projection q | k | v (``with_kv``) or q alone (followed by ``more_columns`` columns that
+    another reader takes), adds the bias, turns pair (i, i + r) of every
     query and key head by position * qk_freqs[i] (r = len(qk_freqs); the coordinates from 2 r on pass), turns the
     value heads the same way over all their coordinates if ``v_freqs`` is given, stores keys and values at the
     step's slots and returns q as [tokens, heads, head_dim]. Angles are taken in float from the position: no table."""
     T = qkv.shape[0]
     width = num_heads * head_dim + (num_kv_heads * (head_dim + value_dim) if with_kv else 0)
-    _dense(qkv, "rotary_split_write: qkv", (T, width))
+    _need(more_columns >= 0, "rotary_split_write: a negative number of further columns")
+    _dense(qkv, "rotary_split_write: qkv", (T, width + more_columns))
     dtype_code(qkv)
     if bias is not None:
         _dense(bias, "rotary_split_write: bias", (width,), qkv.dtype)
@@ -1457,7 +1521,8 @@ def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: t
     if T:
         backend().rotary_split_write(qkv, bias, qk_freqs, rot, v_freqs if with_kv else None, positions,
                                      slot_mapping if with_kv else None, q_out, k_cache if with_kv else None,
-                                     v_cache if with_kv else None, num_heads, num_kv_heads, head_dim, value_dim, with_kv)
+                                     v_cache if with_kv else None, num_heads, num_kv_heads, head_dim, value_dim, with_kv,
+                                     **({"more_columns": int(more_columns)} if more_columns else {}))
     return q_out
 
 
@@ -1473,30 +1538,41 @@ def turn_back_(x: torch.Tensor, freqs: torch.Tensor, positions: torch.Tensor) ->
     return x
 
 
-def gated_delta_rule(proj: torch.Tensor, a_lin: torch.Tensor, gate_lin: torch.Tensor, taps: torch.Tensor,
+def gated_delta_rule(proj: torch.Tensor, a_lin: torch.Tensor | None, gate_lin: torch.Tensor | None, taps: torch.Tensor,
                      dt_bias: torch.Tensor, a_log: torch.Tensor, norm_weight: torch.Tensor, eps: float,
                      kept: torch.Tensor, state: torch.Tensor, batch: AttentionBatch, state_slots: torch.Tensor,
-                     num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, out_dtype) -> torch.Tensor:
+                     num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, out_dtype,
+                     decay_per_head: bool = False, gate_activation: str = "sigmoid") -> torch.Tensor:
     """The recurrent mixer between its projections: short causal convolutions and SiLU on q, k, v (``proj``:
-    [tokens, q | k | v | beta] as projected; ``taps`` [channels, n]; ``kept`` [slots, channels, n - 1], a request's
+    [tokens, q | k | v | beta ...] as projected; ``taps`` [channels, n]; ``kept`` [slots, channels, n - 1], a request's
     last inputs, updated here), unit length for q and k per head, beta = sigmoid, the decays
-    exp(-exp(a_log) softplus(a_lin + dt_bias)) per head and key channel, the recurrence over every request's tokens in
+    exp(-exp(a_log) softplus(a_lin + dt_bias)) per head and key channel (``decay_per_head``: one per head, and then
+    ``a_lin`` has a column and ``dt_bias`` an entry per head), the recurrence over every request's tokens in
     order from and into ``state`` [slots, heads, value_dim, head_dim] (a request whose first token is at position 0
     starts from zero), then per head the read-out over its root mean square times ``norm_weight`` times
-    sigmoid(gate_lin). Returns [tokens, heads * value_dim] in ``out_dtype``. ``a_lin`` is overwritten."""
+    f(gate_lin), f = ``gate_activation`` ("sigmoid", or "silu": z sigmoid(z)). Returns [tokens, heads * value_dim]
+    in ``out_dtype``. ``a_lin`` is overwritten with the decays. ``a_lin`` and ``gate_lin`` None: ``proj`` is float32
+    and holds them as further columns, q | k | v | beta | a | gate (one product made them all)."""
     T = proj.shape[0]
     H, G, D, E = num_heads, num_kv_heads, head_dim, value_dim
     C = 2 * G * D + H * E
+    Dd = 1 if decay_per_head else D
     _need(H % G == 0, lambda: f"gated_delta_rule: {H} heads are not a multiple of {G} key heads")
-    _dense(proj, "gated_delta_rule: proj", (T, C + H))
-    dtype_code(proj)
-    _float32(a_lin, "gated_delta_rule: decays' linear part", (T, H * D))
-    _float32(gate_lin, "gated_delta_rule: gates' linear part", (T, H * E))
+    _need(gate_activation in ("sigmoid", "silu"), lambda: f"gated_delta_rule: gate activation {gate_activation!r}")
+    _need((a_lin is None) == (gate_lin is None), "gated_delta_rule: decays and gates come both packed or both apart")
+    packed = a_lin is None
+    if packed:
+        _dense(proj, "gated_delta_rule: proj", (T, C + H + H * Dd + H * E), torch.float32)
+    else:
+        _dense(proj, "gated_delta_rule: proj", (T, C + H))
+        dtype_code(proj)
+        _float32(a_lin, "gated_delta_rule: decays' linear part", (T, H * Dd))
+        _float32(gate_lin, "gated_delta_rule: gates' linear part", (T, H * E))
     _need(taps.dim() == 2 and taps.shape[0] == C and 1 <= taps.shape[1] <= 16,
           lambda: f"gated_delta_rule: taps {tuple(taps.shape)} for {C} channels (1 to 16 taps)")
     _dense(taps, "gated_delta_rule: taps", dtype=torch.float32)
     n = taps.shape[1]
-    _float32(dt_bias, "gated_delta_rule: dt_bias", (H * D,))
+    _float32(dt_bias, "gated_delta_rule: dt_bias", (H * Dd,))
     _float32(a_log, "gated_delta_rule: a_log", (H,))
     _float32(norm_weight, "gated_delta_rule: norm weight", (E,))
     _need(kept.dim() == 3 and tuple(kept.shape[1:]) == (C, n - 1), lambda: f"gated_delta_rule: kept inputs {tuple(kept.shape)}")
@@ -1521,11 +1597,135 @@ def gated_delta_rule(proj: torch.Tensor, a_lin: torch.Tensor, gate_lin: torch.Te
     if T == 0:
         return y
     b = backend()
-    b.delta_prepare(proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E)
+    act = {"gate_act": 1} if gate_activation == "silu" else {}
+    if packed:
+        decay = torch.empty((T, H, Dd), dtype=torch.float32, device=dev)
+        b.delta_prepare(proj, taps, kept, proj, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E, decay=decay,
+                        a_col=C + H)
+    elif decay_per_head:
+        decay = a_lin.view(T, H, 1)
+        b.delta_prepare(proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E, decay=decay)
+    else:
+        decay = a_lin.view(T, H, D)
+        b.delta_prepare(proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E)
     b.conv_state_update(proj, kept, n, batch, state_slots, C)
-    b.delta_rule(q, k, v, a_lin.view(T, H, D), beta, state, o, batch, state_slots)
-    b.gated_head_norm(o, gate_lin.view(T, H, E), norm_weight, y.view(T, H, E), float(eps))
+    b.delta_rule(q, k, v, decay, beta, state, o, batch, state_slots)
+    if packed:
+        b.gated_head_norm(o, proj, norm_weight, y.view(T, H, E), float(eps), gate_col=C + H + H * Dd, **act)
+    else:
+        b.gated_head_norm(o, gate_lin, norm_weight, y.view(T, H, E), float(eps), **act)
     return y
+
+
+# ------------------------------------------------------------------ several residual streams side by side
+@dataclass
+class ScaledPairSum:
+    """sa a + sb b of two mixers' results that is still to be taken: ``streams_step`` takes it as the sublayer's
+    result and does the sum in its own kernel; ``tensor()`` is the same as a tensor, for any other reader."""
+
+    a: torch.Tensor
+    sa: float
+    b: torch.Tensor
+    sb: float
+
+    def tensor(self) -> torch.Tensor:
+        _dense(self.a, "scaled sum: a")
+        _dense(self.b, "scaled sum: b", tuple(self.a.shape), self.a.dtype)
+        dtype_code(self.a)
+        y = torch.empty_like(self.a)
+        if y.numel():
+            backend().scaled_sum(self.a, self.b, y, float(self.sa), float(self.sb))
+        return y
+
+
+def streams_step(streams: torch.Tensor | None, rows: int, width: int, n: int, rows_dtype, start: torch.Tensor | None = None,
+                 update: tuple | None = None, read: tuple | None = None, collapse: bool = False):
+    """One step of ``n`` residual streams [n, rows, width] (float32) between two sublayers.
+    ``start`` [rows, width] float32: all streams equal it (``streams`` is then only written, or None with ``collapse``).
+    ``update`` = (mix [n, n] (from, to), out [n], y): X_t <- sum_s mix[s, t] X_s + out[t] y, all at once from the old
+    values; y: rows of ``rows_dtype`` or a ``ScaledPairSum`` of two such. (mix and out None: ones, for n = 1.)
+    ``read`` = (in [n] or None for ones, norm weight [width], eps): returns the RMS norm of sum_s in[s] X_s (new values)
+    times the weight, in ``rows_dtype``.
+    ``collapse``: the sum of the (new) streams is returned as [rows, width] float32 and ``streams`` is not written.
+    Returns (normed rows or None, sum or None)."""
+    _need(1 <= n <= 16, lambda: f"streams_step: {n} streams (1 to 16 are taken)")
+    _need(rows_dtype in _DTYPE_CODE, lambda: f"streams_step: rows of {rows_dtype}")
+    if streams is not None:
+        _dense(streams, "streams_step: streams", (n, rows, width), torch.float32)
+    else:
+        _need(start is not None and collapse, "streams_step: without streams there is a start and only a sum is wanted")
+    if start is not None:
+        _dense(start, "streams_step: start", (rows, width), torch.float32)
+    dev = start.device if start is not None else streams.device
+    mix = out_w = a = b = None
+    sa = sb = 1.0
+    if update is not None:
+        mix, out_w, y = update
+        if mix is None:
+            _need(n == 1, "streams_step: several streams need their coefficients")
+            mix, out_w = _ones(dev, 1).view(1, 1), _ones(dev, 1)
+        _float32(mix, "streams_step: mix", (n, n))
+        _float32(out_w, "streams_step: out", (n,))
+        if isinstance(y, ScaledPairSum):
+            a, sa, b, sb = y.a, float(y.sa), y.b, float(y.sb)
+            _dense(b, "streams_step: the second result", (rows, width), rows_dtype)
+        else:
+            a = y
+        _dense(a, "streams_step: the sublayer's result", (rows, width), rows_dtype)
+    in_w = norm_w = h = None
+    eps = 0.0
+    if read is not None:
+        in_w, norm_w, eps = read
+        if in_w is not None:
+            _float32(in_w, "streams_step: in", (n,))
+        _float32(norm_w, "streams_step: norm weight", (width,))
+        h = torch.empty((rows, width), dtype=rows_dtype, device=dev)
+    total = torch.empty((rows, width), dtype=torch.float32, device=dev) if collapse else None
+    _need(update is not None or read is not None or collapse or start is not None, "streams_step: nothing to do")
+    if rows:
+        backend().streams_step(streams, start, mix, out_w, a, b, sa, sb, in_w, norm_w, float(eps), h, total, n, rows, width,
+                               rows_dtype)
+    return h, total
+
+
+_ONES: dict = {}
+
+
+def _ones(device, n: int) -> torch.Tensor:
+    key = (str(device), n)
+    if key not in _ONES:
+        _ONES[key] = torch.ones(n, dtype=torch.float32, device=device)
+    return _ONES[key]
+
+
+def embed_float(ids: torch.Tensor, table: torch.Tensor, scale: float | None = None) -> torch.Tensor:
+    """Rows of ``table`` times ``scale`` as float32 [tokens, width] (the start of a float32 stream: nothing is rounded)."""
+    _need(table.dim() == 2, "embed_float: the table must be [vocab, width]")
+    _dense(table, "embed_float: table")
+    _dense(ids, "embed_float: ids", (ids.shape[0],), torch.int32)
+    dtype_code(table)
+    out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=table.device)
+    if ids.shape[0]:
+        backend().embed_float(ids, table, out, 1.0 if scale is None else float(scale))
+    return out
+
+
+def activation_(x: torch.Tensor, activation: str) -> torch.Tensor:
+    """x <- act(x) in place, taken in float and rounded once; ``activation``: one of ``PLAIN_ACTIVATIONS``."""
+    _need(activation in PLAIN_ACTIVATIONS, lambda: f"activation: {activation!r} is not known ({sorted(PLAIN_ACTIVATIONS)} are)")
+    _dense(x, "activation: x")
+    dtype_code(x)
+    if x.numel():
+        backend().activation(x, PLAIN_ACTIVATIONS[activation])
+    return x
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """x <- x * factor in place (float32)."""
+    _dense(x, "scale: x", dtype=torch.float32)
+    if x.numel():
+        backend().scale(x, float(factor))
+    return x
 
 
 def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

@@ -176,3 +176,102 @@ class ParallelTwoNormsBlock(Part):
         else:
             ops.add_streams_(hidden, mixed, fed)
         return hidden, None
+
+
+@BLOCKS.register("stream_mix")
+class StreamMixBlock(Part):
+    """A pre-norm layer on ``streams`` residual streams X_1 .. X_n (hyper-connections). For each sublayer q (the
+    mixer, then the feed-forward) with coefficients in_q [n], mix_q [n, n] (from, to) and out_q [n]:
+        u = sum_s in_q[s] X_s;   y = sublayer(norm_q(u));   X_t <- sum_s mix_q[s, t] X_s + out_q[t] y,
+    all streams at once from their old values. Before the first such block all streams equal the embedding's rows;
+    after the last their sum goes on. ``learned`` False: one stream with coefficients of 1, which is the plain
+    pre-norm layer x <- x + sublayer(norm(x)) on a float32 stream. The streams are float32 and are what the block
+    takes and returns as ``hidden`` ([n, tokens, width]; the first block takes [tokens, width], the last returns
+    that). One kernel stands between two sublayers: it takes the result of the one into the streams and reads the
+    next one's input through its norm, also across the border to the next block. The feed-forward may be absent."""
+
+    norm_slots = ("mixer_norm", "feed_forward_norm")
+    norms_ahead = True            # the model tells the block which block follows (``next_norm`` is that block's ``norm``)
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, streams: int = 1, learned: bool = True):
+        if not 1 <= streams <= 16:
+            raise ValueError(f"1 to 16 streams are taken, got {streams}")
+        if not learned and streams != 1:
+            raise ValueError("several streams need coefficients")
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.streams, self.learned = streams, bool(learned)
+        self.row_dtype = None
+
+    @property
+    def norm(self):
+        """What the block before this one is shown as the norm that takes its result: this block itself (its first
+        sublayer's coefficients and norm are read in that block's last kernel)."""
+        return self
+
+    def children(self):
+        out = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.feed_forward is not None:
+            out["feed_forward_norm"] = self.feed_forward_norm
+            out["feed_forward"] = self.feed_forward
+        return out
+
+    def param_specs(self):
+        if not self.learned:
+            return {}
+        n = self.streams
+
+        def three(q):
+            return {f"{q}.in": ParamSpec((n,), always_float32=True, init_mean=1.0 / n, init_std=0.1),
+                    f"{q}.mix": ParamSpec((n, n), always_float32=True, init_mean=1.0 / n, init_std=0.1),
+                    f"{q}.out": ParamSpec((n,), always_float32=True, init_mean=1.0, init_std=0.1)}
+        return dict(three("hc1"), **(three("hc2") if self.feed_forward is not None else {}))
+
+    def bind(self, params):
+        self.coefficients = {}
+        for q in ("hc1", "hc2"):
+            if f"{q}.in" in params:
+                self.coefficients[q] = (params[f"{q}.in"], params[f"{q}.mix"], params[f"{q}.out"])
+            else:
+                self.coefficients[q] = (None, None, None)
+
+    def _read(self, q: str, norm) -> tuple:
+        return (self.coefficients[q][0], norm.weight, norm.eps)
+
+    def first_read(self) -> tuple:
+        """What the kernel before this block's mixer reads: (in, norm weight, eps)."""
+        return self._read("hc1", self.mixer_norm)
+
+    def forward(self, hidden, residual, step, cache, next_norm=None):
+        if residual is not None:
+            raise ValueError("this block carries its streams itself and takes no residual beside them")
+        n, dtype = self.streams, self.row_dtype or torch.float32
+        ahead = step.scratch.pop("stream_rows_ahead", None)
+        if hidden.dim() == 2:                      # the first block: all streams start as the embedding's rows
+            if hidden.dtype != torch.float32:
+                hidden = hidden.float()
+            T, W = hidden.shape
+            X = torch.empty((n, T, W), dtype=torch.float32, device=hidden.device)
+            h, _ = ops.streams_step(X, T, W, n, dtype, start=hidden, read=self.first_read())
+        else:
+            X = hidden
+            _, T, W = X.shape
+            if ahead is not None and ahead[0] is self and ahead[1] is X:
+                h = ahead[2]                       # the block before has read this block's first input already
+            else:
+                h, _ = ops.streams_step(X, T, W, n, dtype, read=self.first_read())
+        defer = {"deferred": True} if getattr(self.mixer, "defers_pair_sum", False) else {}
+        y = self.mixer.forward(h, step, cache, **defer)
+        _, mix, out = self.coefficients["hc1"]
+        if self.feed_forward is not None:
+            h, _ = ops.streams_step(X, T, W, n, dtype, update=(mix, out, y), read=self._read("hc2", self.feed_forward_norm))
+            y = self.feed_forward.forward(h, step)
+            _, mix, out = self.coefficients["hc2"]
+        if isinstance(next_norm, StreamMixBlock) and next_norm.streams == n:
+            h, _ = ops.streams_step(X, T, W, n, dtype, update=(mix, out, y), read=next_norm.first_read())
+            step.scratch["stream_rows_ahead"] = (next_norm, X, h)
+            return X, None
+        if next_norm is not None:
+            raise ValueError("a block of several streams is followed by a block of its kind and its number of streams")
+        _, total = ops.streams_step(X, T, W, n, dtype, update=(mix, out, y), collapse=True)
+        return total, None

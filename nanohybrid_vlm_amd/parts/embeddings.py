@@ -30,3 +30,14 @@ class HashedPairEmbedding(Part):
     def forward(self, step, table: torch.Tensor, state: dict) -> torch.Tensor:
         return ops.embed_pair_hash(step.input_ids, table, self.pair_weight, step.attention, step.state_slots,
                                    state["prev"], self.buckets, self.mul_prev, self.mul_cur)
+
+
+@EMBEDDINGS.register("scaled_float")
+class ScaledFloatEmbedding(Part):
+    """x_t = table[token_t] * scale as float32: the start of a float32 stream, multiplied and kept unrounded."""
+
+    def __init__(self, scale: float | None = None):
+        self.scale = None if scale is None else float(scale)
+
+    def forward(self, step, table: torch.Tensor, state) -> torch.Tensor:
+        return ops.embed_float(step.input_ids, table, self.scale)

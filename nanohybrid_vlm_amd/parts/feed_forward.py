@@ -42,6 +42,27 @@ class SwiGLU(Part):
         return ops.linear(ops.gated_linear(x, self.gate_up_weight), self.down_weight, add_to=add_to)
 
 
+@FEED_FORWARDS.register("plain_mlp")
+class PlainMLP(Part):
+    """down(act(up(x))) without a gate and without biases; ``activation``: "relu2" (the square of max(z, 0)), "silu"
+    or "gelu_tanh". The activation is taken in float on the up projection's rows and rounded once."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2"):
+        if activation not in ops.PLAIN_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not known ({sorted(ops.PLAIN_ACTIVATIONS)} are)")
+        if min(hidden_size, intermediate_size) <= 0:
+            raise ValueError(f"a feed-forward of {hidden_size} x {intermediate_size}")
+        self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
+        self.up_weight = self.down_weight = None
+
+    def param_specs(self):
+        return {"up.weight": ParamSpec((self.intermediate_size, self.hidden_size)),
+                "down.weight": ParamSpec((self.hidden_size, self.intermediate_size))}
+
+    def forward(self, x, step):
+        return ops.linear(ops.activation_(ops.linear(x, self.up_weight), self.activation), self.down_weight)
+
+
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(Part):
     """``num_experts`` gated feed-forwards of inner size ``expert_size`` without biases, of which every token uses the

@@ -92,11 +92,14 @@ class RotaryAttention(Part):
     value at position j is stored turned by j over all its coordinates (pairs (m, m + value_dim / 2), frequencies of
     the encoding's base over value_dim, unscaled), and each head's result at position i is turned back by i.
     ``own_kv`` False: the layer has no key and value projections and reads the cache of the run-order entry it
-    borrows from (keys as stored, after rotation) with queries, mask and output projection of its own."""
+    borrows from (keys as stored, after rotation) with queries, mask and output projection of its own.
+    ``softcap`` c: a score s (after the scale) becomes c tanh(s / c). ``sink`` z: the softmax's denominator holds one
+    more term exp(z), a key of that score that has no value. ``head_gate``: head h's result is multiplied by
+    sigmoid(w_h . x), x the mixer's input; the rows w_h are the last ``num_heads`` rows of the packed projection."""
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
                  bias: bool, position, chunk: int | None = None, window: int | None = None, rotate_values: bool = False,
-                 own_kv: bool = True):
+                 own_kv: bool = True, softcap: float | None = None, sink: float | None = None, head_gate: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} key/value heads")
         if window and chunk:
@@ -107,6 +110,11 @@ class RotaryAttention(Part):
         self.head_dim, self.value_dim, self.scale, self.bias = head_dim, value_dim, scale, bias
         self.position, self.chunk, self.window = position, chunk or None, window or None
         self.rotate_values, self.own_kv = rotate_values, own_kv
+        if softcap is not None and not softcap > 0:
+            raise ValueError(f"a cap on the scores must be positive, got {softcap}")
+        if head_gate and bias:
+            raise ValueError("a gate per head and biases are not taken together")
+        self.softcap, self.sink, self.head_gate = softcap, sink, bool(head_gate)
         self.qkv_weight = self.qkv_bias = self.o_weight = None
 
     def _packed_width(self) -> int:
@@ -116,7 +124,8 @@ class RotaryAttention(Part):
         return width
 
     def param_specs(self):
-        specs = {"qkv.weight": ParamSpec((self._packed_width(), self.hidden_size)),
+        gates = self.num_heads if self.head_gate else 0
+        specs = {"qkv.weight": ParamSpec((self._packed_width() + gates, self.hidden_size)),
                  "o.weight": ParamSpec((self.hidden_size, self.num_heads * self.value_dim))}
         if self.bias:
             specs["qkv.bias"] = ParamSpec((self._packed_width(),), init="zeros")
@@ -136,15 +145,22 @@ class RotaryAttention(Part):
         if not self.own_kv and cache.writes:
             raise ValueError("an attention layer without key and value projections must borrow another entry's cache")
         qkv = ops.linear(x, self.qkv_weight)
+        gates = self.num_heads if self.head_gate else 0
         if self.own_kv and not writes:               # a layer with projections of its own that reads a lent cache
+            if gates:
+                raise ValueError("a layer with a gate per head and projections of its own cannot read a lent cache")
             qkv = qkv[:, :self.num_heads * self.head_dim].contiguous()
         bias = self.qkv_bias if (self.qkv_bias is None or writes or not self.own_kv) else \
             self.qkv_bias[:self.num_heads * self.head_dim].contiguous()
         freqs = self.position.frequencies() if self.position is not None and self.position.rotary_dim else None
         v_freqs = self.position.frequencies_for(self.value_dim) if self.rotate_values else None
         q = ops.rotary_split_write(qkv, bias, freqs, v_freqs, step.token_positions, tables.slot_mapping, cache.k, cache.v,
-                                   self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, with_kv=writes)
-        o = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window, self.chunk)
+                                   self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, with_kv=writes,
+                                   more_columns=gates)
+        # (the gates stay where the projection left them: the attention kernels read them from the packed rows)
+        o = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window, self.chunk,
+                                softcap=self.softcap, sink=self.sink,
+                                gate=(qkv, qkv.shape[1] - gates) if gates else None)
         if self.rotate_values:
             ops.turn_back_(o, v_freqs, step.token_positions)
         return ops.linear(o.view(o.shape[0], self.num_heads * self.value_dim), self.o_weight)
@@ -161,27 +177,46 @@ class GatedDeltaRule(Part):
     head and key channel; the read-out is divided by its root mean square per head (``eps``), multiplied by a weight
     over value_dim and by sigmoid(W_g2 W_g1 x), and projected. The state and the last taps - 1 inputs of the
     convolutions live in the request's state slot; a request that starts at position 0 starts from zeros.
-    ``decay_rank``, ``gate_rank``: the inner sizes of the two low-rank projections."""
+    ``decay_rank``, ``gate_rank``: the inner sizes of the two low-rank projections; both None: the decays' and the
+    gates' linear parts are plain projections of x, rows of the one packed input projection (q | k | v | beta | a | g).
+    ``decay_per_head``: one decay per head (a projection row and a ``dt_bias`` entry per head) in place of one per head
+    and key channel. ``gate_activation``: "sigmoid", or "silu" (the read-out times g sigmoid(g))."""
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, conv_taps: int,
-                 decay_rank: int, gate_rank: int, eps: float, position=None):
+                 decay_rank: int | None, gate_rank: int | None, eps: float, position=None, decay_per_head: bool = False,
+                 gate_activation: str = "sigmoid"):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} key heads")
         if not 1 <= conv_taps <= 16:
             raise ValueError(f"1 to 16 taps are taken, got {conv_taps}")
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
         self.head_dim, self.value_dim, self.conv_taps = head_dim, value_dim, conv_taps
+        if (decay_rank is None) != (gate_rank is None):
+            raise ValueError("the decays' and the gates' projections are both low-rank or both plain")
+        if gate_activation not in ("sigmoid", "silu"):
+            raise ValueError(f"gate activation {gate_activation!r} is not known ('sigmoid' and 'silu' are)")
         self.decay_rank, self.gate_rank, self.eps = decay_rank, gate_rank, eps
+        self.decay_per_head, self.gate_activation = bool(decay_per_head), gate_activation
+        self.decay_dim = 1 if decay_per_head else head_dim
         self.channels = 2 * num_kv_heads * head_dim + num_heads * value_dim
 
     def param_specs(self):
         H, D, E, W = self.num_heads, self.head_dim, self.value_dim, self.hidden_size
+        if self.decay_rank is None:
+            return {
+                "in.weight": ParamSpec((self.channels + H + H * self.decay_dim + H * E, W)),     # q | k | v | beta | a | g
+                "conv.weight": ParamSpec((self.channels, self.conv_taps), always_float32=True, init_mean=0.0, init_std=0.5),
+                "dt_bias": ParamSpec((H * self.decay_dim,), always_float32=True, init_mean=-1.0, init_std=1.0),
+                "A_log": ParamSpec((H,), always_float32=True, init_mean=-1.0, init_std=0.5),
+                "norm.weight": ParamSpec((E,), init="norm", always_float32=True),
+                "o.weight": ParamSpec((W, H * E)),
+            }
         return {
             "in.weight": ParamSpec((self.channels + H, W)),                  # q | k | v | beta
             "conv.weight": ParamSpec((self.channels, self.conv_taps), always_float32=True, init_mean=0.0, init_std=0.5),
             "a1.weight": ParamSpec((self.decay_rank, W)),
-            "a2.weight": ParamSpec((H * D, self.decay_rank)),
-            "dt_bias": ParamSpec((H * D,), always_float32=True, init_mean=-1.0, init_std=1.0),
+            "a2.weight": ParamSpec((H * self.decay_dim, self.decay_rank)),
+            "dt_bias": ParamSpec((H * self.decay_dim,), always_float32=True, init_mean=-1.0, init_std=1.0),
             "A_log": ParamSpec((H,), always_float32=True, init_mean=-1.0, init_std=0.5),
             "g1.weight": ParamSpec((self.gate_rank, W)),
             "g2.weight": ParamSpec((H * E, self.gate_rank)),
@@ -195,11 +230,14 @@ class GatedDeltaRule(Part):
 
     def forward(self, x, step, cache: CacheView):
         proj = ops.linear(x, self.in_weight, out_dtype=torch.float32)
-        a_lin = ops.linear(ops.linear(x, self.a1_weight), self.a2_weight, out_dtype=torch.float32)
-        g_lin = ops.linear(ops.linear(x, self.g1_weight), self.g2_weight, out_dtype=torch.float32)
+        a_lin = g_lin = None                     # (plain projections: further columns of ``proj``)
+        if self.decay_rank is not None:
+            a_lin = ops.linear(ops.linear(x, self.a1_weight), self.a2_weight, out_dtype=torch.float32)
+            g_lin = ops.linear(ops.linear(x, self.g1_weight), self.g2_weight, out_dtype=torch.float32)
         y = ops.gated_delta_rule(proj, a_lin, g_lin, self.conv_weight, self.dt_bias, self.A_log, self.norm_weight, self.eps,
                                  cache.state["kept"], cache.state["S"], step.attention, step.state_slots, self.num_heads,
-                                 self.num_kv_heads, self.head_dim, self.value_dim, x.dtype)
+                                 self.num_kv_heads, self.head_dim, self.value_dim, x.dtype,
+                                 decay_per_head=self.decay_per_head, gate_activation=self.gate_activation)
         return ops.linear(y, self.o_weight)
 
 
@@ -222,17 +260,7 @@ class NormedPair(Part):
                 "right_out.weight": ParamSpec((self.hidden_size,), init="norm", always_float32=True)}
 
     def cache_need(self):
-        paged = state = None
-        for need in (self.left.cache_need(), self.right.cache_need()):
-            if isinstance(need, PagedKVNeed):
-                if paged is not None:
-                    raise ValueError("two mixers side by side cannot both keep pages")
-                paged = need
-            elif isinstance(need, StateNeed):
-                if state is not None:
-                    raise ValueError("two mixers side by side cannot both keep state")
-                state = need
-        return CombinedNeed(paged, state)
+        return _side_by_side_need(self.left, self.right)
 
     defers_pair_norm = True       # ``forward(..., deferred=True)`` may return an ``ops.NormedPairMean``
 
@@ -242,4 +270,47 @@ class NormedPair(Part):
         a = self.left.forward(x, step, cache)
         b = self.right.forward(x, step, cache)
         pair = ops.NormedPairMean(a, self.left_out_weight, b, self.right_out_weight, self.eps)
+        return pair if deferred else pair.tensor()
+
+
+def _side_by_side_need(left, right):
+    """What two mixers side by side need together: at most one of them keeps pages and at most one keeps state."""
+    paged = state = None
+    for need in (left.cache_need(), right.cache_need()):
+        if isinstance(need, PagedKVNeed):
+            if paged is not None:
+                raise ValueError("two mixers side by side cannot both keep pages")
+            paged = need
+        elif isinstance(need, StateNeed):
+            if state is not None:
+                raise ValueError("two mixers side by side cannot both keep state")
+            state = need
+    return CombinedNeed(paged, state)
+
+
+@MIXERS.register("scaled_pair")
+class ScaledPair(Part):
+    """Two mixers side by side that read the same rows: ``left_scale`` times the left one's result plus
+    ``right_scale`` times the right one's. One of them may keep pages and the other state."""
+
+    def __init__(self, left: dict, right: dict, left_scale: float, right_scale: float, position=None, **offered):
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+        self.left = MIXERS.build(left, offered=offered, position=position)
+        self.right = MIXERS.build(right, offered=offered, position=position)
+        self.recordable = self.left.recordable and self.right.recordable
+
+    def children(self):
+        return {"left": self.left, "right": self.right}
+
+    def cache_need(self):
+        return _side_by_side_need(self.left, self.right)
+
+    defers_pair_sum = True        # ``forward(..., deferred=True)`` may return an ``ops.ScaledPairSum``
+
+    def forward(self, x, step, cache: CacheView, deferred: bool = False):
+        """``deferred``: the caller's next step is a kernel that takes the two results with their sum still to do
+        (``ops.streams_step``); it then gets an ``ops.ScaledPairSum`` in place of a tensor."""
+        a = self.left.forward(x, step, cache)
+        b = self.right.forward(x, step, cache)
+        pair = ops.ScaledPairSum(a, self.left_scale, b, self.right_scale)
         return pair if deferred else pair.tensor()

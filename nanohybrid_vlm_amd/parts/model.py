@@ -63,6 +63,7 @@ class ModelSpec:
     eos_token_id: int | None = None           # the token that ends a request, if the checkpoint names one
     embed_scale: float | None = None          # the embedding's rows are multiplied by this (in float, then rounded)
     logit_cap: float | None = None            # logits become cap * tanh(logits / cap)
+    logit_scale: float | None = None          # logits are multiplied by this (in float, before any cap)
     position_axes: int = 1                    # coordinates of a token's position (a step carries [axes, tokens])
     embed_norm: dict | None = None            # a norm that the embedding's rows pass before the first layer
     embedding: dict | None = None             # None: the rows of the table; else a registered embedding that uses the table
@@ -235,6 +236,8 @@ class DecoderModel(Part):
     def logits(self, hidden: torch.Tensor) -> torch.Tensor:
         """float32 logits [n, vocab] (the reference's sampler casts to float first, nanovllm/layers/sampler.py:12)."""
         logits = ops.linear(hidden, self.head_weight, out_dtype=torch.float32)
+        if self.spec.logit_scale is not None and self.spec.logit_scale != 1.0:
+            ops.scale_(logits, self.spec.logit_scale)
         if self.spec.logit_cap is not None:
             ops.soft_cap_(logits, self.spec.logit_cap)
         return logits

@@ -100,3 +100,26 @@ class LayerNorm(Part):
             x = x.float()
         y, _ = ops.layernorm_pair(x, (self.weight, self.bias), None, self.eps, out_dtype or self.row_dtype or torch.float32)
         return y
+
+
+@NORMS.register("stream_rmsnorm")
+class StreamRMSNorm(Part):
+    """y = x / sqrt(mean(x^2) + eps) * weight of a float32 stream, given as rows of the model's element type;
+    statistics and weight are float32. A block that carries several streams reads this norm's weight and eps and
+    takes the norm in its own kernel (``ops.streams_step``); ``forward`` is the same for one stream."""
+
+    def __init__(self, size: int, eps: float):
+        self.size, self.eps = size, eps
+        self.weight = None
+        self.row_dtype = None         # set when the model's weights are bound
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.size,), init="norm", always_float32=True)}
+
+    def forward(self, x, out_dtype=None) -> torch.Tensor:
+        if x.dtype != torch.float32:
+            x = x.float()
+        rows, width = x.shape
+        y, _ = ops.streams_step(x.view(1, rows, width), rows, width, 1, out_dtype or self.row_dtype or torch.float32,
+                                read=(None, self.weight, self.eps))
+        return y

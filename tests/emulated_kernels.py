@@ -7,6 +7,8 @@ product: the engine never selects it; only tests install it with
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 
@@ -78,7 +80,8 @@ class EmulatedBackend:
             k_cache.view(-1, Hkv, D)[slots] = k[ok]
             v_cache.view(-1, Hkv, D)[slots] = v[ok].to(dt)
 
-    def paged_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window, chunk=0):
+    def paged_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window, chunk=0, cap=0.0, sink=None,
+                        gate=None):
         T, Hq, D = q.shape
         page_size, Hkv = k_cache.shape[1], k_cache.shape[2]
         group = Hq // Hkv
@@ -96,7 +99,17 @@ class EmulatedBackend:
                 kh = kf[slots, h // group].float()
                 vh = vf[slots, h // group].float()
                 s = (kh @ q[t, h].float()) * scale
-                out[t, h] = (torch.softmax(s, dim=0) @ vh).to(out.dtype)
+                if cap:
+                    s = cap * torch.tanh(s / cap)
+                if sink is None:
+                    o = torch.softmax(s, dim=0) @ vh
+                else:
+                    m = max(float(s.max()), sink)
+                    e = torch.exp(s - m)
+                    o = (e @ vh) / (e.sum() + math.exp(sink - m))
+                if gate is not None:
+                    o = o * torch.sigmoid(gate[0][t, gate[1] + h].float())
+                out[t, h] = o.to(out.dtype)
 
     # -- layers that are not the pre-norm kind
     def scalar_rmsnorm(self, x, gain, y, eps):
@@ -242,9 +255,11 @@ class EmulatedBackend:
         return torch.cat((u * cos - v * sin, v * cos + u * sin, t[..., 2 * half:]), dim=-1)
 
     def rotary_split_write(self, qkv, bias, qk_freqs, rot, v_freqs, positions, slot_mapping, q_out, k_cache, v_cache,
-                           Hq, Hkv, D, E, with_kv):
+                           Hq, Hkv, D, E, with_kv, more_columns=0):
         T, dt = qkv.shape[0], qkv.dtype
         x = qkv.float()
+        if more_columns:
+            x = x[:, :x.shape[1] - more_columns]
         if bias is not None:
             x = (x + bias.float()).to(dt).float()
         q = x[:, :Hq * D].reshape(T, Hq, D)
@@ -265,8 +280,11 @@ class EmulatedBackend:
         x.copy_(self._turned(x.float(), positions, freqs, sign=-1.0).to(x.dtype))
 
     # -- the gated delta rule: the four kernels, request by request and token by token
-    def delta_prepare(self, proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E):
+    def delta_prepare(self, proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E,
+                      decay=None, a_col=0):
         n = taps.shape[1]
+        Dd = D if decay is None else decay.shape[2]
+        into = a_lin if decay is None else decay.view(proj.shape[0], H * Dd)
         C = 2 * G * D + H * E
         x = proj.float()
         for t in range(proj.shape[0]):
@@ -285,9 +303,9 @@ class EmulatedBackend:
             q[t] = qk[:G] * D ** -0.5
             k[t] = qk[G:]
             v[t] = act[2 * G * D:].view(H, E)
-            step = torch.nn.functional.softplus(a_lin[t] + dt_bias, threshold=20.0)
-            a_lin[t] = torch.exp(-torch.exp(a_log).repeat_interleave(D) * step)
-            beta[t] = torch.sigmoid(x[t, C:])
+            step = torch.nn.functional.softplus(a_lin[t, a_col:a_col + H * Dd] + dt_bias, threshold=20.0)
+            into[t] = torch.exp(-torch.exp(a_log).repeat_interleave(Dd) * step)
+            beta[t] = torch.sigmoid(x[t, C:C + H])
 
     def conv_state_update(self, proj, kept, n_taps, batch, state_slots, channels):
         x = proj.float()
@@ -324,9 +342,48 @@ class EmulatedBackend:
                     out[t, h] = S @ q[t, g]
                 state[slot, h] = S
 
-    def gated_head_norm(self, o, gate, w, y, eps):
+    def gated_head_norm(self, o, gate, w, y, eps, gate_col=0, gate_act=0):
+        T, H, E = o.shape
+        z = gate[:, gate_col:gate_col + H * E].reshape(T, H, E)
         r = torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
-        y.copy_((o * r * w * torch.sigmoid(gate)).to(y.dtype))
+        y.copy_((o * r * w * (z * torch.sigmoid(z) if gate_act == 1 else torch.sigmoid(z))).to(y.dtype))
+
+    # -- several residual streams side by side
+    def streams_step(self, X, x0, mix, out_w, a, b, sa, sb, in_w, norm_w, eps, h, total, n, T, W, rows_dtype):
+        old = x0[None].expand(n, T, W) if x0 is not None else X
+        if mix is not None:
+            y = sa * a.float()
+            if b is not None:
+                y = y + sb * b.float()
+            new = torch.einsum("st,srw->trw", mix, old) + out_w[:, None, None] * y[None]
+        else:
+            new = old.clone()
+        if total is not None:
+            total.copy_(new.sum(0))
+        elif mix is not None or x0 is not None:
+            X.copy_(new)
+        if h is not None:
+            u = new.sum(0) if in_w is None else torch.einsum("s,srw->rw", in_w, new)
+            h.copy_((u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * norm_w).to(h.dtype))
+
+    def embed_float(self, ids, table, out, scale):
+        out.copy_(table[ids.long()].float() * scale)
+
+    def activation(self, x, act):
+        z = x.float()
+        if act == 0:
+            z = z * torch.sigmoid(z)
+        elif act == 1:
+            z = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        else:
+            z = torch.clamp(z, min=0.0) ** 2
+        x.copy_(z.to(x.dtype))
+
+    def scaled_sum(self, a, b, y, sa, sb):
+        y.copy_((sa * a.float() + sb * b.float()).to(y.dtype))
+
+    def scale(self, x, factor):
+        x.mul_(factor)
 
     def linear(self, x, w, bias, out):
         y = x.float() @ w.float().T

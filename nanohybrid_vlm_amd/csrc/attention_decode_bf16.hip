@@ -16,6 +16,10 @@
 // key positions. Each split writes its unnormalised output with (maximum, sum) in
 // float; a second kernel merges the splits in rising order. Keys that are not visible
 // are loaded as zeros (the cache's unused slots may hold anything).
+// What a layer may ask for besides (the entry point ..._more): a cap on the scores (s <- cap tanh(s / cap), after the
+// scale; taken on the float scores where they leave the first product), one more term exp(sink) in the softmax's
+// denominator (it joins in the merge, as a split without values would) and a gate per (token, head) whose sigmoid
+// multiplies the head's result (in the merge, with the division by the sum).
 #include "nhv_common.h"
 #include "nhv_no_alloc.h"
 #include <math.h>
@@ -57,11 +61,14 @@ __device__ __forceinline__ int slot_of(const int* bt, int key, int page_size, in
   return bt[key / page_size] * page_size + key % page_size;
 }
 
+// CAPPED: the scores pass cap tanh(s scale / cap). cap_l2 = cap log2(e); tanh_k = 2 log2(e) scale / cap, so that
+// tanh(x) = 1 - 2 / (1 + exp(2 x)) costs one exp2 and one reciprocal (an overflowing exp2 gives the limit 1).
+template <bool CAPPED>
 __global__ __launch_bounds__(64) void decode_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     float* __restrict__ part_o, float* __restrict__ part_ml, const int* __restrict__ token_req,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv,
-    int page_size, int page_shift, float scale_log2e, int window, int split_len, int n_splits) {
+    int page_size, int page_shift, float scale_log2e, int window, int split_len, int n_splits, float cap_l2, float tanh_k) {
   __shared__ __attribute__((aligned(16))) bf16_t vt_s[D * VPITCH];
   const int lane = threadIdx.x;
   // blocks go to the eight XCDs in turn by their linear index: with the split as the slowest index every XCD
@@ -161,7 +168,10 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int key = kb + kt * 16 + grp * 4 + j;
-        const float v = (key >= first && key <= last) ? s4[kt][j] * scale_log2e : -INFINITY;
+        float scaled = s4[kt][j] * scale_log2e;
+        if (CAPPED)
+          scaled = __builtin_fmaf(-2.0f * cap_l2, __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(s4[kt][j] * tanh_k)), cap_l2);
+        const float v = (key >= first && key <= last) ? scaled : -INFINITY;
         s4[kt][j] = v;
         m_tile = fmaxf(m_tile, v);
       }
@@ -243,7 +253,8 @@ constexpr int MPIECES = (MQ + MLPR - 1) / MLPR;             // pieces per lane (
 template <int W>
 __global__ __launch_bounds__(64 * W) void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                               bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                              int window, int split_len, int n_splits, int Hq) {
+                                                              int window, int split_len, int n_splits, int Hq, float sink_l2,
+                                                              const bf16_t* __restrict__ gate, long long gate_ld) {
   __shared__ float4 sum_s[W > 1 ? W - 1 : 1][MPIECES][64];
   const int item = blockIdx.x;               // t * Hq + h
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -259,8 +270,9 @@ __global__ __launch_bounds__(64 * W) void merge_splits_kernel(const float* __res
   m = wave_max(m);
   float l = 0.f;
   for (int s = s0 + lane; s <= s1; s += 64) l += ml[s * 2 + 1] * exp2f(ml[s * 2] - m);
-  l = wave_sum(l);
-  const float inv = 1.0f / l;
+  l = wave_sum(l) + exp2f(sink_l2 - m);       // (no sink: sink_l2 is -inf and the term 0)
+  float inv = 1.0f / l;
+  if (gate) inv /= 1.0f + expf(-(float)gate[(size_t)t * gate_ld + item % Hq]);
   const float* po = part_o + (size_t)item * n_splits * D;
   const int sub = lane / MLPR, piece = lane % MLPR;
   float4 acc[MPIECES];
@@ -323,7 +335,8 @@ template <int W, int NL>
 __global__ __launch_bounds__(64 * W) void merge_splits_at_once_kernel(const float* __restrict__ part_o,
                                                                       const float* __restrict__ part_ml,
                                                                       bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                                      int window, int split_len, int n_splits, int Hq) {
+                                                                      int window, int split_len, int n_splits, int Hq, float sink_l2,
+                                                                      const bf16_t* __restrict__ gate, long long gate_ld) {
   __shared__ float4 sum_s[W > 1 ? W - 1 : 1][MPIECES][64];
   __shared__ float ml_s[W > 1 ? W - 1 : 1][2];
   const int item = blockIdx.x;               // t * Hq + h
@@ -358,6 +371,7 @@ __global__ __launch_bounds__(64 * W) void merge_splits_at_once_kernel(const floa
   for (int off = MLPR; off < 64; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
   const float m_ref = m == -INFINITY ? 0.f : m;          // a wave none of whose splits the position reaches
   float l = 0.f;
+  float m_final = m_ref;                                 // what the sums are taken against in the end
   float4 acc[MPIECES];
 #pragma unroll
   for (int p = 0; p < MPIECES; ++p) acc[p] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -393,6 +407,7 @@ __global__ __launch_bounds__(64 * W) void merge_splits_at_once_kernel(const floa
 #pragma unroll
     for (int wv = 0; wv < W - 1; ++wv) m_all = fmaxf(m_all, ml_s[wv][0]);
     const float own = exp2f(m - m_all);                    // (some split is reached, so m_all is a number)
+    m_final = m_all;
     l *= own;
 #pragma unroll
     for (int p = 0; p < MPIECES; ++p) { acc[p].x *= own; acc[p].y *= own; acc[p].z *= own; acc[p].w *= own; }
@@ -408,7 +423,9 @@ __global__ __launch_bounds__(64 * W) void merge_splits_at_once_kernel(const floa
     }
   }
   if (sub == 0) {
-    const float inv = 1.0f / l;
+    l += exp2f(sink_l2 - m_final);                         // (no sink: sink_l2 is -inf and the term 0)
+    float inv = 1.0f / l;
+    if (gate) inv /= 1.0f + expf(-(float)gate[(size_t)(item / Hq) * gate_ld + item % Hq]);
 #pragma unroll
     for (int p = 0; p < MPIECES; ++p) {
       const int qd = piece + p * MLPR;
@@ -427,18 +444,26 @@ extern "C" int nhv_decode_attention_head_dim() { return D; }
 static int launch_decode_attention(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_o,
                                    float* part_ml, const void* token_req, const void* positions,
                                    const void* block_tables, int max_blocks, int T, int Hq, int Hkv, int page_size,
-                                   float scale, int window, int split_len, int n_splits, hipStream_t s) {
+                                   float scale, int window, int split_len, int n_splits, hipStream_t s, float cap = 0.f,
+                                   int has_sink = 0, float sink = 0.f, const void* gate = nullptr, long long gate_ld = 0) {
   int page_shift = -1;
   for (int b = 0; b < 31; ++b)
     if (page_size == (1 << b)) page_shift = b;
   dim3 grid(Hkv, T, n_splits);
-  hipLaunchKernelGGL(decode_attention_kernel, grid, dim3(64), 0, s, (const bf16_t*)q, (const bf16_t*)k_cache,
-                     (const bf16_t*)v_cache, part_o, part_ml, (const int*)token_req,
-                     (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, page_shift,
-                     scale * 1.4426950408889634f, window, split_len, n_splits);
+  const float log2e = 1.4426950408889634f;
+#define NHV_DECODE_LAUNCH(CAPPED_)                                                                                    \
+  hipLaunchKernelGGL(decode_attention_kernel<CAPPED_>, grid, dim3(64), 0, s, (const bf16_t*)q, (const bf16_t*)k_cache, \
+                     (const bf16_t*)v_cache, part_o, part_ml, (const int*)token_req,                                  \
+                     (const int*)positions, (const int*)block_tables, max_blocks, Hq, Hkv, page_size, page_shift,     \
+                     scale * log2e, window, split_len, n_splits, cap * log2e, cap > 0.f ? 2.0f * log2e * scale / cap : 0.f)
+  if (cap > 0.f) NHV_DECODE_LAUNCH(true);
+  else NHV_DECODE_LAUNCH(false);
+#undef NHV_DECODE_LAUNCH
   NHV_LAUNCH_CHECK("decode_attention");
   const unsigned items = (unsigned)((size_t)T * Hq);
-#define NHV_MERGE_ARGS (const float*)part_o, (const float*)part_ml, (bf16_t*)out, (const int*)positions, window, split_len, n_splits, Hq
+  const float sink_l2 = has_sink ? sink * log2e : -INFINITY;
+#define NHV_MERGE_ARGS (const float*)part_o, (const float*)part_ml, (bf16_t*)out, (const int*)positions, window, split_len, n_splits, Hq, \
+                       sink_l2, (const bf16_t*)gate, gate_ld
 #define NHV_MERGE_AT_ONCE(W_, NL_) \
   hipLaunchKernelGGL((merge_splits_at_once_kernel<W_, NL_>), dim3(items), dim3(64 * W_), 0, s, NHV_MERGE_ARGS)
   // few splits: everything asked for at once, by four waves from the point where one wave's lanes would take more
@@ -481,6 +506,20 @@ extern "C" int nhv_decode_attention_bf16(const void* q, const void* k_cache, con
   return launch_decode_attention(q, k_cache, v_cache, out, (float*)part_o, (float*)part_ml, token_req, positions,
                                  block_tables, max_blocks, T, Hq, Hkv, page_size, scale, window, split_len, n_splits,
                                  (hipStream_t)stream);
+}
+
+// The same with a cap on the scores (0: none), one more term exp(sink) in the denominator (has_sink) and a gate per
+// (token, head): gate[t * gate_ld + h] in bfloat16, whose sigmoid multiplies the head's result (null: none).
+extern "C" int nhv_decode_attention_bf16_more(const void* q, const void* k_cache, const void* v_cache, void* out, void* part_o,
+                                              void* part_ml, const void* token_req, const void* positions,
+                                              const void* block_tables, int max_blocks, int T, int Hq, int Hkv, int page_size,
+                                              float scale, int window, int split_len, int n_splits, float cap, int has_sink,
+                                              float sink, const void* gate, long long gate_ld, void* stream) {
+  if (check_decode_attention(max_blocks, T, Hq, Hkv, page_size, window, split_len, n_splits)) return 1;
+  NHV_REQUIRE(cap >= 0.f && (!gate || gate_ld >= Hq), "decode attention: cap %g, gate rows %lld apart for %d heads", (double)cap, gate_ld, Hq);
+  return launch_decode_attention(q, k_cache, v_cache, out, (float*)part_o, (float*)part_ml, token_req, positions,
+                                 block_tables, max_blocks, T, Hq, Hkv, page_size, scale, window, split_len, n_splits,
+                                 (hipStream_t)stream, cap, has_sink, sink, gate, gate_ld);
 }
 
 // ---- the entry point that allocates nothing (nhv_no_alloc.h) ----

@@ -34,6 +34,10 @@
 // comes as a negative window, else 0). Keys outside the block's range are replaced by the
 // nearest key inside it (their P is 0): unused cache slots may hold anything, and 0 * NaN
 // would poison the sums.
+// What a layer may ask for besides (MORE; the entry point ..._more): a cap on the scores (s <- cap tanh(s / cap), after
+// the scale; taken on the float scores where they leave the first product), one more term exp(sink) in the softmax's
+// denominator (it joins the row's sum at the end, against the row's reference point) and a gate per (token, head) whose
+// sigmoid multiplies the head's result (with the division by the sum).
 #include "nhv_common.h"
 #include <math.h>
 #include <type_traits>
@@ -86,12 +90,16 @@ __device__ __forceinline__ int slot_of(P bt, int key, int page_size, int page_sh
 
 // BT_IN_LDS: the request's block table (up to the block's last key) is copied into LDS first, so that the
 // look-up that every load of a key depends on costs an LDS read instead of a trip to memory.
-template <bool BT_IN_LDS, int RT>
+// MORE: cap_ratio = cap / scale (0: no cap) and tanh_k = 2 log2(e) scale / cap, so that the capped score, still to be
+// multiplied by the scale as every score is, costs one exp2 and one reciprocal: tanh(x) = 1 - 2 / (1 + exp(2 x)), and an
+// exp2 that overflows gives the limit 1; sink_l2 = sink log2(e), or -inf for none; gate (may be null).
+template <bool BT_IN_LDS, int RT, bool MORE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void prefill_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens_q, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, int max_blocks, int Hq, int Hkv, int page_size, int page_shift,
-    float scale_log2e, int window) {
+    float scale_log2e, int window, float cap_ratio, float tanh_k, float sink_l2, const bf16_t* __restrict__ gate,
+    long long gate_ld) {
   constexpr int DL = SUPPORTED ? D : 16;                   // keeps the unsupported sizes compilable; they are never launched
   constexpr int TILE = SUPPORTED ? BN * DL : 16;           // elements of a tile
   __shared__ __attribute__((aligned(16))) bf16_t k_s0[TILE], k_s1[TILE], v_s0[TILE], v_s1[TILE];
@@ -250,6 +258,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
         for (int r = 0; r < RT; ++r) s4[r][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[r][s], s4[r][kt], 0, 0, 0);
       }
     }
+    if (MORE && cap_ratio > 0.f) {
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            s4[r][kt][j] = __builtin_fmaf(-2.0f * cap_ratio,
+                                          __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(s4[r][kt][j] * tanh_k)), cap_ratio);
+    }
     bf16x8 pa[RT][KT / 2];                                 // P of keys (32 a + 4 grp + j) and (32 a + 16 + 4 grp + j)
     float alpha[RT];
     bool grow[RT];
@@ -367,7 +385,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (row_ok[r]) {
-      const float inv = 1.0f / l;
+      if (MORE) l += __builtin_amdgcn_exp2f(sink_l2 - m_run[r]);      // (a row that is stored has seen its own key: m_run is a number)
+      float inv = 1.0f / l;
+      if (MORE && gate) inv /= 1.0f + expf(-(float)gate[(size_t)(q_begin + row_tok[r]) * gate_ld + head[r]]);
       bf16_t* dst = out + ((size_t)(q_begin + row_tok[r]) * Hq + head[r]) * D;
 #pragma unroll
       for (int dt = 0; dt < DTILES; ++dt) {
@@ -382,10 +402,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
 
 }  // namespace prefill
 
-extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                          const void* cu_seqlens_q, const void* context_lens, const void* block_tables,
-                                          int max_blocks, int B, int max_q_len, int Hq, int Hkv, int page_size, float scale,
-                                          int window, void* stream) {
+static int launch_prefill_attention(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                    const void* cu_seqlens_q, const void* context_lens, const void* block_tables,
+                                    int max_blocks, int B, int max_q_len, int Hq, int Hkv, int page_size, float scale,
+                                    int window, void* stream, bool more, float cap, int has_sink, float sink, const void* gate,
+                                    long long gate_ld) {
   NHV_REQUIRE(B > 0 && max_q_len > 0 && Hq > 0 && Hkv > 0 && page_size > 0 && max_blocks > 0, "prefill attention: bad sizes");
   NHV_REQUIRE(Hq % Hkv == 0, "prefill attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   NHV_REQUIRE(prefill::SUPPORTED, "prefill attention: head size %d is beyond this kernel's limit of 256", prefill::D);
@@ -400,11 +421,20 @@ extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, co
   const int tpb = two ? 8 : 4;
   const long long gx = (row_tiles + tpb - 1) / tpb;
   NHV_REQUIRE(gx <= 0x7fffffff && Hkv <= 65535 && B <= 65535, "prefill attention: grid too large");
-#define NHV_PREFILL_LAUNCH(BT, RT_)                                                                                    \
-  hipLaunchKernelGGL((prefill::prefill_attention_kernel<BT, RT_>), dim3((unsigned)gx, Hkv, B), dim3(256), 0,         \
+  const float log2e = 1.4426950408889634f;
+  const bool capped = more && cap > 0.f;
+#define NHV_PREFILL_LAUNCH_AS(BT, RT_, MORE_)                                                                          \
+  hipLaunchKernelGGL((prefill::prefill_attention_kernel<BT, RT_, MORE_>), dim3((unsigned)gx, Hkv, B), dim3(256), 0,  \
                      (hipStream_t)stream, (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, \
                      (const int*)cu_seqlens_q, (const int*)context_lens, (const int*)block_tables, max_blocks, Hq, Hkv, \
-                     page_size, page_shift, scale * 1.4426950408889634f, window)
+                     page_size, page_shift, scale * log2e, window, capped ? cap / scale : 0.f,                         \
+                     capped ? 2.0f * log2e * scale / cap : 0.f, more && has_sink ? sink * log2e : -INFINITY,           \
+                     (const bf16_t*)gate, gate_ld)
+#define NHV_PREFILL_LAUNCH(BT, RT_)            \
+  do {                                         \
+    if (more) NHV_PREFILL_LAUNCH_AS(BT, RT_, true); \
+    else NHV_PREFILL_LAUNCH_AS(BT, RT_, false);     \
+  } while (0)
   const bool bt_in_lds = max_blocks <= prefill::BT_LDS;
   if (two) {
     if (bt_in_lds) NHV_PREFILL_LAUNCH(true, prefill::MAX_RT);
@@ -414,6 +444,28 @@ extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, co
     else NHV_PREFILL_LAUNCH(false, 1);
   }
 #undef NHV_PREFILL_LAUNCH
+#undef NHV_PREFILL_LAUNCH_AS
   NHV_LAUNCH_CHECK("prefill_attention");
   return 0;
+}
+
+extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                          const void* cu_seqlens_q, const void* context_lens, const void* block_tables,
+                                          int max_blocks, int B, int max_q_len, int Hq, int Hkv, int page_size, float scale,
+                                          int window, void* stream) {
+  return launch_prefill_attention(q, k_cache, v_cache, out, cu_seqlens_q, context_lens, block_tables, max_blocks, B, max_q_len,
+                                  Hq, Hkv, page_size, scale, window, stream, false, 0.f, 0, 0.f, nullptr, 0);
+}
+
+// The same with a cap on the scores (0: none; a positive scale is then needed), one more term exp(sink) in the
+// denominator (has_sink) and a gate per (token, head): gate[t * gate_ld + h] in bfloat16 (null: none).
+extern "C" int nhv_prefill_attention_bf16_more(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                               const void* cu_seqlens_q, const void* context_lens, const void* block_tables,
+                                               int max_blocks, int B, int max_q_len, int Hq, int Hkv, int page_size,
+                                               float scale, int window, float cap, int has_sink, float sink, const void* gate,
+                                               long long gate_ld, void* stream) {
+  NHV_REQUIRE(cap >= 0.f && (cap == 0.f || scale > 0.f) && (!gate || gate_ld >= Hq),
+              "prefill attention: cap %g with scale %g, gate rows %lld apart for %d heads", (double)cap, (double)scale, gate_ld, Hq);
+  return launch_prefill_attention(q, k_cache, v_cache, out, cu_seqlens_q, context_lens, block_tables, max_blocks, B, max_q_len,
+                                  Hq, Hkv, page_size, scale, window, stream, true, cap, has_sink, sink, gate, gate_ld);
 }

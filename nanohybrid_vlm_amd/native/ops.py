@@ -193,13 +193,14 @@ class NativeBackend:
         _, page_size, Hkv, _ = k_cache.shape
         E = v_cache.shape[3]
         plain = not cap and sink is None and gate is None
+        more = () if plain else (ctypes.c_float(cap or 0.0), int(sink is not None), ctypes.c_float(sink or 0.0), *_gate_args(gate))
         # the kernels on the matrix cores take value heads of the key heads' size; a chunk goes to them as a negative window
-        fast = plain and q.dtype == torch.bfloat16 and E == D and D % 16 == 0 and D <= 256
+        fast = q.dtype == torch.bfloat16 and E == D and D % 16 == 0 and D <= 256
         if chunk:
             window = -chunk
         if fast and batch.max_q_len == 1 and Hq // Hkv <= 16 and T <= 65535:
-            return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window)
-        if fast and batch.max_q_len == 1 and Hkv == 1 and T <= 65535:
+            return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window, more)
+        if fast and plain and batch.max_q_len == 1 and Hkv == 1 and T <= 65535:
             # more than 16 query heads on one key/value head (a cached latent): sixteen heads at a time
             for h0 in range(0, Hq, 16):
                 part = torch.empty((T, min(16, Hq - h0), E), dtype=out.dtype, device=out.device)
@@ -208,10 +209,10 @@ class NativeBackend:
             return None
         if fast and batch.num_requests <= 65535 and Hkv <= 65535:
             # prompt portions (and whatever single tokens share their batch) on the matrix cores
-            return self._call("nhv_prefill_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
-                              _ptr(batch.cu_seqlens_q), _ptr(batch.context_lens), _ptr(block_tables),
+            return self._call("nhv_prefill_attention_bf16" + ("_more" if more else ""), _ptr(q), _ptr(k_cache), _ptr(v_cache),
+                              _ptr(out), _ptr(batch.cu_seqlens_q), _ptr(batch.context_lens), _ptr(block_tables),
                               block_tables.shape[1], batch.num_requests, batch.max_q_len, Hq, Hkv, page_size,
-                              ctypes.c_float(scale), window, _stream(), lib=self.attention_lib(D))
+                              ctypes.c_float(scale), window, *more, _stream(), lib=self.attention_lib(D))
         self._call("nhv_paged_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
                    _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables), block_tables.shape[1], T, Hq, Hkv,
                    D, E, page_size, ctypes.c_float(scale), 0 if chunk else window, chunk, ctypes.c_float(cap or 0.0),
@@ -399,8 +400,9 @@ class NativeBackend:
         self._call("nhv_experts_down", _ptr(u), _ptr(ids), _ptr(down), _ptr(out), T, W, F, ids.shape[1], E,
                    dtype_code(u), _stream())
 
-    def _decode_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window):
-        """Single tokens in bfloat16: keys split over waves, then merged."""
+    def _decode_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window, more=()):
+        """Single tokens in bfloat16: keys split over waves, then merged. ``more``: the arguments of a cap on the
+        scores, a further term in the denominator and a gate per head, for the entry point that takes them."""
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
         # inside a graph the lengths are only bounded (by max_model_len): the recorder says what to plan for
@@ -428,10 +430,10 @@ class NativeBackend:
         n_splits = -(-covered // split_len)
         part_o = torch.empty((T, Hq, n_splits, D), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, Hq, n_splits, 2), dtype=torch.float32, device=q.device)
-        self._call("nhv_decode_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_o),
-                   _ptr(part_ml), _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables),
+        self._call("nhv_decode_attention_bf16" + ("_more" if more else ""), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
+                   _ptr(part_o), _ptr(part_ml), _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables),
                    block_tables.shape[1], T, Hq, Hkv, page_size, ctypes.c_float(scale), window, split_len, n_splits,
-                   _stream(), lib=self.attention_lib(D))
+                   *more, _stream(), lib=self.attention_lib(D))
 
     # -- matrix products of few rows: own kernel or one of the library's algorithms, by measurement --
     def blas_lib(self) -> ctypes.CDLL:

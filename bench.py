@@ -19,9 +19,9 @@ For these two ``value`` is generated tokens a second over the whole run, prompts
 ``--workload projections`` is a diagnosis, not the benchmark: a layer's matrix products alone, cold, beside a kernel
 that only reads the same bytes (see ``bench_projections``).
 
-``--workload design --shape pevazen-1b|pevazen-8b|fazovik-1b|fazovik-8b [--layers L]``: a model of the Pevazen or the Fazovik design (attention and
-recurrent layers side by side, see ``architectures/pevazen.py``) beside a Qwen3 model of the same width, heads,
-feed-forward size, vocabulary and number of layers: one prompt of ``--prompt-tokens`` in one step, decoding at
+``--workload design --shape pevazen-1b|pevazen-8b|fazovik-1b|fazovik-8b|vugelix-1b|vugelix-8b [--layers L]``: a model of the Pevazen, the
+Fazovik or the Vugelix design (see ``architectures/``) beside a Qwen3 model (for Vugelix: a Pevazen model of pairs of
+mixers) of the same width, heads, feed-forward size, vocabulary and number of layers: one prompt of ``--prompt-tokens`` in one step, decoding at
 ``--batch`` requests, and the time of every own kernel in one eager step of each kind (see ``bench_design``).
 """
 import argparse
@@ -422,12 +422,26 @@ def bench_design(args):
     from nanohybrid_vlm_amd.engine.runner import StepEntry
     from nanohybrid_vlm_amd.native import ops
 
-    name = args.shape if args.shape.startswith(("pevazen", "fazovik")) else "pevazen-1b"
+    name = args.shape if args.shape.startswith(("pevazen", "fazovik", "vugelix")) else "pevazen-1b"
     design = name.split("-")[0]
     new = json.loads(json.dumps(named_shapes()[name]))
     layers = args.layers or min(8, len(new["layers"]))
     new["layers"] = new["layers"][:layers]
-    if design == "fazovik":
+    beside = "qwen3"
+    if design == "vugelix":
+        # the closest model the engine has is Pevazen's pair of mixers (attention beside a gated delta rule): the twin is
+        # made of such layers alone, with this design's heads and head sizes on both sides, a chunk as long as the
+        # window, and a (gated) feed-forward of the same inner size
+        beside = "pevazen"
+        entries = []
+        for layer in new["layers"]:
+            a, r = layer["mixer"]["left"], layer["mixer"]["right"]
+            left = {"dim": a["dim"], "heads": a["heads"], "kv_heads": a["kv_heads"], "mask": {"size": a["mask"]["size"]},
+                    "rot": {"base": a["rot"]["base"], "dims": a["dim"]}, "scale": a["scale"], "vdim": a["vdim"]}
+            right = dict(r, decay_rank=128, gate_rank=128)
+            entries.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": layer["mlp"]})
+        twin = {"architecture": "Pevazen", "layers": entries, "norm": {"eps": 1e-6}, "vocab": new["vocab"], "width": new["width"]}
+    elif design == "fazovik":
         # the twin has as many heads, of the size of this design's value heads, a quarter as many key/value heads, and
         # the dense layers' inner size in every layer
         a = new["layers"][0]["mixer"]
@@ -440,7 +454,7 @@ def bench_design(args):
     context = args.context or (T + 512)
     pages = (batch + 1) * -(-context // args.block_size) + 1
     out = {}
-    for label, raw in ((design, new), ("qwen3", twin)):
+    for label, raw in ((design, new), (beside, twin)):
         llm = LLM(raw, random_weights=0, dtype=args.dtype, kvcache_block_size=args.block_size, max_num_seqs=max(batch, 1),
                   enforce_eager=args.eager, num_kvcache_blocks=pages, max_num_batched_tokens=max(args.token_budget, T, batch),
                   max_model_len=context, scheduler_policy="prefill_first")
@@ -487,13 +501,13 @@ def bench_design(args):
         llm.exit()
         del llm, runner
         torch.cuda.empty_cache()
-    line = {"metric": f"{design.capitalize()} ({name}, {layers} layers) beside Qwen3 of equal sizes: prefill of {T} tokens and decode at batch {batch}",
+    line = {"metric": f"{design.capitalize()} ({name}, {layers} layers) beside {beside.capitalize()} of equal sizes: prefill of {T} tokens and decode at batch {batch}",
             "value": out[design]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": out[design]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random token ids, random weights",
             "config": {"model": name, "layers": layers, "width": new["width"], "global_batch": batch, "prompt_len": T,
                        "seq_len": context, "parallelism": "single GPU", "graphs": not args.eager},
-            design: out[design], "qwen3": out["qwen3"]}
+            design: out[design], beside: out[beside]}
     print(json.dumps(line), flush=True)
     return 0
 

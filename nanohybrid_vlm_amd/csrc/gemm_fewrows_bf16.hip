@@ -219,6 +219,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* 
     float r = v[0][j] * rs;
     if (bias && n < N) r += (float)bias[n];
     if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
+    else if (f.plain_act) r = nhv_plain_act(r, f.plain_act);
     out[j] = r;
   }
   emit_tile<FUSED, TOut>(f, out, y, col, grp, n0 + nt * 16, blockIdx.x * NT + nt, (N + 15) / 16, M, N);
@@ -345,6 +346,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
       float r = v[0][j] * rs;
       if (bias && n < N) r += (float)bias[n];
       if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
+      else if (f.plain_act) r = nhv_plain_act(r, f.plain_act);
       out[j] = r;
     }
     emit_tile<FUSED && !GLU, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N, res_ahead);
@@ -449,6 +451,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const b
       float r = v[0][j] * rs;
       if (bias && n < N) r += (float)bias[n];
       if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
+      else if (f.plain_act) r = nhv_plain_act(r, f.plain_act);
       out[j] = r;
     }
     emit_tile<FUSED, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N);
@@ -561,6 +564,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_passes_kernel(const b
         float r = v[0][j] * rs;
         if (bias && n < N) r += (float)bias[n];
         if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
+        else if (f.plain_act) r = nhv_plain_act(r, f.plain_act);
         out[j] = r;
       }
       emit_tile<FUSED, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N);

@@ -192,6 +192,19 @@ extern "C" int nhv_gemm_fewrows_glu_act_bf16(const void* x, const void* w, void*
   return 0;
 }
 
+// y = act(x . w^T) for up to 16 rows: the first half of a feed-forward without a gate in one kernel. act: 1 SiLU, 2 the
+// tanh form of GELU, 3 the square of max(z, 0); taken in float on the finished sums and rounded once.
+extern "C" int nhv_gemm_fewrows_act_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype, int act,
+                                         void* stream) {
+  if (sk_check("few-rows gemm with activation", x, w, M, N, K, out_dtype)) return 1;
+  NHV_REQUIRE(M <= 16 && act >= 1 && act <= 3, "few-rows gemm with activation: %d rows (up to 16), activation %d", M, act);
+  NhvGemmFusion f = {};
+  f.plain_act = act;
+  if (nhv_gemm_fewrows_launch(false, x, w, nullptr, y, M, N, K, out_dtype, (hipStream_t)stream, f)) return 1;
+  NHV_LAUNCH_CHECK("gemm_fewrows_act_bf16");
+  return 0;
+}
+
 // ---- products of up to 16 rows that take over the kernels around them (nhv_gemm_fusion.h) ----
 // y = r . (x . w^T) (+ bias), or with glu silu(r . (x . w[0:N]^T)) * (r . (x . w[N:2N]^T)), for 1 <= M <= 16 rows in
 // bfloat16. With ss_in: x is a sum (times its norm's weight) whose rows still lack their scales: r per row from ss_in

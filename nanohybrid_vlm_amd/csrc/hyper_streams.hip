@@ -10,15 +10,17 @@
 //  - nhv_embed_float: rows of the table times a scale, as floats (the start of a float stream).
 //  - nhv_activation: an activation on rows, in place.  nhv_scale: float numbers times one number, in place.
 //  - nhv_scaled_sum: sa a + sb b of two tensors of rows.
-// One block per token; a thread owns columns i, i + 256, ...; the sum over a row's squares is taken in an order that
+// One block per token, of 256, 512 or 1,024 threads by the width alone (a step of a few single tokens is a few blocks,
+// and what it takes is the chain of loads and stores of one thread: at most four columns a thread from a width of
+// 1,024 on); a thread owns columns i, i + threads, ...; the sum over a row's squares is taken in an order that
 // depends on the width only, so a token's result does not depend on its batch.
 #include "nhv_common.h"
 #include <math.h>
 
 #define NHV_MAX_STREAMS 16
 
-template <typename TR, int NMAX>
-__global__ __launch_bounds__(256) void streams_step_kernel(
+template <typename TR, int NMAX, int THREADS>
+__global__ __launch_bounds__(THREADS) void streams_step_kernel(
     float* __restrict__ X, long long stride, const float* __restrict__ x0, const float* __restrict__ mix,
     const float* __restrict__ out_w, const TR* __restrict__ a, const TR* __restrict__ b, float sa, float sb,
     const float* __restrict__ in_w, const float* __restrict__ norm_w, float eps, TR* __restrict__ h,
@@ -97,10 +99,16 @@ extern "C" int nhv_streams_step(void* X, long long stride, const void* x0, const
   const size_t lds = ((size_t)W + 16 + (size_t)n * n + 2 * n) * sizeof(float);
   NHV_REQUIRE(lds <= 64 * 1024, "streams_step: a width of %d does not fit the kernel's 64 KB of LDS", W);
   hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(TR, NMAX)                                                                                             \
-  hipLaunchKernelGGL((streams_step_kernel<TR, NMAX>), dim3(T), dim3(256), lds, s, (float*)X, stride, (const float*)x0, \
-                     (const float*)mix, (const float*)out_w, (const TR*)a, (const TR*)b, sa, sb, (const float*)in_w,  \
-                     (const float*)norm_w, eps, (TR*)h, (float*)total, n, W)
+#define LAUNCH_AS(TR, NMAX, THREADS)                                                                                  \
+  hipLaunchKernelGGL((streams_step_kernel<TR, NMAX, THREADS>), dim3(T), dim3(THREADS), lds, s, (float*)X, stride,     \
+                     (const float*)x0, (const float*)mix, (const float*)out_w, (const TR*)a, (const TR*)b, sa, sb,    \
+                     (const float*)in_w, (const float*)norm_w, eps, (TR*)h, (float*)total, n, W)
+#define LAUNCH(TR, NMAX)                             \
+  do {                                               \
+    if (W <= 1024) LAUNCH_AS(TR, NMAX, 256);         \
+    else if (W <= 2048) LAUNCH_AS(TR, NMAX, 512);    \
+    else LAUNCH_AS(TR, NMAX, 1024);                  \
+  } while (0)
 #define BY_N(TR)                                     \
   do {                                               \
     if (n == 1) LAUNCH(TR, 1);                       \
@@ -114,6 +122,7 @@ extern "C" int nhv_streams_step(void* X, long long stride, const void* x0, const
   else return nhv_fail("streams_step: unknown dtype %d", rows_dtype);
 #undef BY_N
 #undef LAUNCH
+#undef LAUNCH_AS
   NHV_LAUNCH_CHECK("streams_step");
   return 0;
 }

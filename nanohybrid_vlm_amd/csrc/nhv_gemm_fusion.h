@@ -22,7 +22,19 @@ struct NhvGemmFusion {
   int tiles_in;
   float eps;
   int glu_act;           // what a gated product passes its gate through: 0 SiLU, 1 the tanh form of GELU
+  int plain_act;         // what a product without a gate passes its result through (after the bias): 0 nothing, 1 SiLU,
+                         // 2 the tanh form of GELU, 3 the square of max(z, 0)
 };
+
+__device__ __forceinline__ float nhv_plain_act(float z, int act) {
+  if (act == 3) {
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+  }
+  if (act == 2) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  if (act == 1) return z / (1.0f + expf(-z));
+  return z;
+}
 
 __device__ __forceinline__ float nhv_glu_gate(float z, int act) {
   if (act == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));

@@ -748,6 +748,20 @@ class NativeBackend:
             return True
         return False
 
+    def activated_linear(self, x, w, out, act: int) -> bool:
+        """act(x W^T) in one kernel, if this batch is one for the few-rows kernel and no library algorithm was found
+        faster for the shape; else False. ``act``: a value of ``PLAIN_ACTIVATIONS``."""
+        M, K = x.shape
+        if not (x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and M <= self.few_rows):
+            return False
+        if not self.own_kernels_only:
+            how = self._choose(x, w, out)
+            if how is not None and how >= 0:
+                return False                                 # the library's product, then the activation's kernel
+        self._call("nhv_gemm_fewrows_act_bf16", _ptr(x), _ptr(w), _ptr(out), M, out.shape[1], K, dtype_code(out), act + 1,
+                   _stream())
+        return True
+
     def sample(self, logits, temperatures, keys, tokens):
         n, V = logits.shape
         pieces = self.lib.nhv_sample_pieces(V)
@@ -1720,6 +1734,24 @@ def activation_(x: torch.Tensor, activation: str) -> torch.Tensor:
     if x.numel():
         backend().activation(x, PLAIN_ACTIVATIONS[activation])
     return x
+
+
+def activated_linear(x: torch.Tensor, w: torch.Tensor, activation: str) -> torch.Tensor:
+    """act(x . w^T) without a gate and without bias: one kernel for few rows in bfloat16, else the matrix product
+    followed by ``activation_``. Either way the activation is taken in float and the result rounded once more than the
+    product alone (the fused kernel rounds once in all)."""
+    _need(activation in PLAIN_ACTIVATIONS, lambda: f"activated_linear: {activation!r} is not known ({sorted(PLAIN_ACTIVATIONS)} are)")
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1],
+          lambda: f"activated_linear: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
+    _dense(x, "activated_linear: x")
+    _dense(w, "activated_linear: w", dtype=x.dtype)
+    dtype_code(x)
+    fused = getattr(backend(), "activated_linear", None)
+    if fused is not None and x.shape[0]:
+        out = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
+        if fused(x, w, out, PLAIN_ACTIVATIONS[activation]):
+            return out
+    return activation_(linear(x, w), activation)
 
 
 def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:

@@ -45,7 +45,8 @@ class SwiGLU(Part):
 @FEED_FORWARDS.register("plain_mlp")
 class PlainMLP(Part):
     """down(act(up(x))) without a gate and without biases; ``activation``: "relu2" (the square of max(z, 0)), "silu"
-    or "gelu_tanh". The activation is taken in float on the up projection's rows and rounded once."""
+    or "gelu_tanh". The activation is taken in float: on the up projection's finished sums where a step of few rows
+    does both in one kernel, else on its rounded rows."""
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2"):
         if activation not in ops.PLAIN_ACTIVATIONS:
@@ -60,7 +61,7 @@ class PlainMLP(Part):
                 "down.weight": ParamSpec((self.hidden_size, self.intermediate_size))}
 
     def forward(self, x, step):
-        return ops.linear(ops.activation_(ops.linear(x, self.up_weight), self.activation), self.down_weight)
+        return ops.linear(ops.activated_linear(x, self.up_weight, self.activation), self.down_weight)
 
 
 @FEED_FORWARDS.register("routed_experts")

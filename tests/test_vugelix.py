@@ -122,6 +122,18 @@ def test_small_kernels(where, kernels):
         ops.activation_(z.clone().to(device), "cube")
     x = torch.randn(4, 9, generator=g)
     assert torch.equal(ops.scale_(x.clone().to(device), 0.25).cpu(), x * 0.25)
+    # a product with its activation: few rows (one kernel in bfloat16 on the GPU) and many
+    wm = (torch.randn(72, 40, generator=g) / 40 ** 0.5 * 2).to(dt)
+    for rows in (1, 5, 16, 33, 200):
+        xm = torch.randn(rows, 40, generator=g).to(dt)
+        for name, fn in (("relu2", plain.squared_relu), ("silu", plain.silu), ("gelu_tanh", None)):
+            got = ops.activated_linear(xm.to(device), wm.to(device), name)
+            z = xm.float() @ wm.float().T
+            want = fn(z) if fn is not None else torch.nn.functional.gelu(z, approximate="tanh")
+            # (many rows in bfloat16: the product's rows are rounded before the activation, which may double their
+            # relative error, and once after it)
+            bound = _tol(dtype, want, coarse=1e-2) + (2.0 ** -6 * want.abs() if dtype == "bfloat16" else 0.0)
+            assert got.dtype == dt and bool(((got.float().cpu() - want).abs() <= bound).all()), (rows, name)
 
 
 def _single_request_batch(T, start, device, page_size, pages):

@@ -321,6 +321,56 @@ def test_delta_rule_with_one_decay_a_head(where, kernels, sizes):
             assert bool(((out - want[r]).abs() <= bound).all()), (round_, r, first_difference(out, want[r], 1e-3))
 
 
+@pytest.mark.parametrize("where", WHERE)
+def test_a_value_written_far_back_is_read_from_the_state(where, kernels):
+    """One token writes a value under a key that no other token uses (its key is the unit vector of channel 0; all other
+    keys have nothing there), with decays of nearly 1. Every later query that asks for channel 0 then reads that value
+    back from the state, hundreds of tokens later, whatever the portions were (the slot held no numbers before); a
+    query before the marked token reads nothing of it. One tap, so the inputs are known."""
+    device, dtype = where
+    H, G, D, E, eps = 2, 1, 8, 6, 1e-6
+    C = 2 * G * D + H * E
+    T, marked = 400, 37
+    g = torch.Generator().manual_seed(4)
+    proj = torch.zeros(T, C + 2 * H + H * E)
+    q_in, k_in = torch.full((T, D), -30.0), 0.5 * torch.randn(T, D, generator=g).abs() + 0.5
+    q_in[:, 0] = 6.0                                         # every query: the unit vector of channel 0
+    k_in[:, 0] = -30.0                                       # no key has anything in channel 0 (SiLU of -30 is nothing) ...
+    k_in[marked] = -30.0
+    k_in[marked, 0] = 6.0                                    # ... but the marked one, which has nothing else
+    v_in = 0.3 * torch.randn(T, H * E, generator=g)
+    v_in[marked] = torch.tensor([3.0, -3.0, 3.0, 3.0, -3.0, -3.0] * H)
+    proj[:, :D], proj[:, D:2 * D], proj[:, 2 * D:C] = q_in, k_in, v_in
+    proj[:, C:C + H] = 8.0                                   # beta: nearly 1
+    proj[:, C + H:C + 2 * H] = -12.0                         # decays: exp(-rate * softplus(-12 + bias)), nearly 1
+    proj[:, C + 2 * H:] = 2.0                                # gates: SiLU(2), the same for every entry
+    taps = torch.ones(C, 1)
+    dt_bias, a_log, norm = torch.zeros(H), torch.zeros(H), torch.ones(E)
+    want = torch.nn.functional.silu(v_in[marked]).view(H, E)         # what the marked token wrote, as the read-out's norm and gate leave it
+    want = want / torch.sqrt(want.pow(2).mean(-1, keepdim=True) + eps) * float(torch.nn.functional.silu(torch.tensor(2.0)))
+    kept = torch.zeros((3, C, 0)).to(device)
+    for portions in ([T], [marked] + [1] * 20 + [T - marked - 20], [2, 33, 5, 1, 1, 200, 1, 1, 156]):
+        state = torch.full((3, H, E, D), float("nan")).to(device)
+        at, outs = 0, []
+        for n in portions:
+            batch = AttentionBatch(num_tokens=n, num_requests=1, token_req=torch.zeros(n, dtype=torch.int32).to(device),
+                                   positions=torch.arange(at, at + n, dtype=torch.int32).to(device),
+                                   cu_seqlens_q=torch.tensor([0, n], dtype=torch.int32).to(device),
+                                   context_lens=torch.tensor([at + n], dtype=torch.int32).to(device), max_q_len=n,
+                                   max_context_len=at + n)
+            y = ops.gated_delta_rule(proj[at:at + n].contiguous().to(device), None, None, taps.to(device), dt_bias.to(device),
+                                     a_log.to(device), norm.to(device), eps, kept, state, batch,
+                                     torch.tensor([1], dtype=torch.int32).to(device), H, G, D, E, _dt(dtype),
+                                     decay_per_head=True, gate_activation="silu")
+            outs.append(y.float().cpu().view(n, H, E))
+            at += n
+        got = torch.cat(outs)
+        # from the marked token on the read-out is the marked value alone; before it nothing is read: zeros
+        close = ((got[marked:] - want).abs() < 0.05).all(-1).all(-1)
+        assert bool(close.all()), (portions, marked + int((~close).nonzero()[0]))
+        assert float(got[:marked].abs().max()) < 1e-2
+
+
 # ------------------------------------------------------------------ configuration and weights
 def test_configuration_and_names(folders):
     from nanohybrid_vlm_amd.parts.base import CombinedNeed

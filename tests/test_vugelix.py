@@ -496,6 +496,32 @@ def test_ways_of_cutting_agree_with_the_plain_model(folders, where, kernels, nam
                 assert torch.equal(results[what][rid], results["whole"][rid]), (what, rid)
 
 
+@pytest.mark.parametrize("where", WHERE)
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(where, kernels, seed, tmp_path):
+    """Models of sizes drawn at random (see ``vugelix_cases.random_config``) in portions, side by side and with a decoded
+    tail, on pages of 16 tokens that are used again, against the plain model; float32 bit-equal across the ways on the GPU."""
+    device, dtype = where
+    cfg = vc.random_config(seed)
+    folder = vc.write_model(str(tmp_path / "m"), cfg, 500 + seed)
+    lengths = [1, 21, 40, 7] if device == "cpu" else [1, 70, 210, 33, 131]
+    requests = {f"r{i}": vc.tokens(cfg["vocab"], n, 7 * i + n) for i, n in enumerate(lengths)}
+    want = _plain_logits(folder, requests)
+    ways = {"portions": vc.in_portions(requests, [17, 2, 3, 64, 1, 33]),
+            "side by side": vc.interleaved(requests, [5, 1, 2, 31, 1, 1, 16], 3),
+            "tail": [s for rid, toks in requests.items() for s in vc.in_portions({rid: toks}, [max(1, len(toks) - 20)] + [1] * 20)]}
+    results = {}
+    for what, steps in ways.items():
+        for i, s in enumerate(steps):
+            s["step"] = i
+        results[what] = _replay(folder, where, steps, page_size=16, max_live=3)
+        _compare(results[what], want, dtype, (seed, what))
+    if device != "cpu" and dtype == "float32":
+        for rid in want:
+            assert torch.equal(results["portions"][rid], results["side by side"][rid]) and \
+                torch.equal(results["portions"][rid], results["tail"][rid]), (seed, rid)
+
+
 @pytest.mark.parametrize("where", ON_GPU)
 def test_pages_of_64_and_windows_longer_than_a_page(folders, where, kernels):
     """Pages of 64 tokens (whole tiles of the prompt kernel lie in one page) under windows of 96 and 160 positions,
@@ -506,6 +532,21 @@ def test_pages_of_64_and_windows_longer_than_a_page(folders, where, kernels):
     for what, steps in (("portions", vc.in_portions(requests, [37, 2, 64, 5, 1, 129, 1, 1, 96])),
                         ("side by side", vc.interleaved(requests, [33, 1, 1, 64, 1, 7, 1, 100], 3))):
         got = _replay(folders["S"], where, steps, page_size=64, max_live=3)
+        _compare(got, want, dtype, what)
+
+
+@pytest.mark.parametrize("where", ON_GPU)
+def test_sizes_of_a_real_models_layers(where, kernels, tmp_path):
+    """Heads and states of 128 and 64 entries, a width of 1,024: the kernels' makes that real sizes take (the streams'
+    kernel with 256 threads a block and more, the products of few rows with their activation, the recurrence with
+    columns of 128), in portions and side by side on pages of 64, with decoded tokens between."""
+    device, dtype = where
+    folder = vc.write_model(str(tmp_path / "w"), vc.CONFIG_W, 26)
+    requests = {f"r{i}": vc.tokens(vc.CONFIG_W["vocab"], n, 11 * i + n) for i, n in enumerate([300, 40, 129])}
+    want = _plain_logits(folder, requests)
+    for what, steps in (("portions", vc.in_portions(requests, [150, 1, 1, 16, 3, 64, 1, 1, 1])),
+                        ("side by side", vc.interleaved(requests, [40, 1, 1, 1, 17, 1, 64, 1], 3))):
+        got = _replay(folder, where, steps, page_size=64, max_live=3)
         _compare(got, want, dtype, what)
 
 

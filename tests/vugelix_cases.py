@@ -75,6 +75,15 @@ CONFIG_S = {
                dict(_S0, weights_of=0)],
 }
 
+# head sizes, state sizes and a width of the kind real models have (two layers and one run again)
+_W0 = _layer(_left(8, 2, 128, 128, 200, 64, 10000.0, 128 ** -0.5 * 2, 20.0), _right(4, 2, 128, 128, 4), 0.6, 0.5, 2048)
+CONFIG_W = {
+    "architecture": "Vugelix", "norm": {"eps": 1e-6}, "vocab": 512, "width": 1024, "streams": 4,
+    "embedding": {"scale": 32.0}, "logit_scale": 0.5,
+    "layers": [_W0, _layer(_left(16, 4, 64, 64, 70, 64, 500000.0, 0.25, 50.0), _right(8, 8, 64, 128, 3), 0.5, 0.5, 3072),
+               dict(_W0, weights_of=0)],
+}
+
 CASES = {"A": (CONFIG_A, 21), "B": (CONFIG_B, 32), "C": (CONFIG_C, 23), "R": (CONFIG_R, 24), "S": (CONFIG_S, 25)}
 
 
@@ -139,3 +148,36 @@ def write_model(folder: str, config: dict, seed: int, tensors: dict | None = Non
     tensors = random_tensors(config, seed) if tensors is None else tensors
     save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
     return folder
+
+
+def random_config(seed: int) -> dict:
+    """A configuration drawn at random (seeded): head sizes that the matrix-core kernels take and sizes that they do
+    not, 1 to 20 query heads per key/value head, widths and vocabularies that are no multiple of 8, 1 to 8 streams or
+    none, windows around the sizes of pages and tiles, layers that run earlier layers' weights in any order."""
+    import random
+    r = random.Random(seed)
+    width = r.choice([24, 40, 52, 64, 72, 100])
+    owners, layers = [], []
+    for i in range(r.randint(2, 5)):
+        if owners and r.random() < 0.4:
+            j = r.choice(owners)
+            layers.append(dict(layers[j], weights_of=j))
+            continue
+        kv = r.choice([1, 2, 3])
+        group = r.choice([1, 2, 4, 5, 17, 20]) if kv == 1 else r.choice([1, 2, 3])
+        dim = r.choice([8, 16, 20, 32, 48, 64])
+        vdim = dim if r.random() < 0.6 else r.choice([4, 12, 16, 24])
+        rot = r.choice([0, 2, dim // 2 // 2 * 2, dim])
+        left = _left(kv * group, kv, dim, vdim, r.choice([1, 3, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 500]), rot,
+                     r.choice([10.0, 1000.0, 50000.0]), r.choice([0.5, 1.0, 2.0]) * dim ** -0.5, r.choice([2.0, 5.0, 30.0]))
+        rkv = r.choice([1, 2])
+        right = _right(rkv * r.choice([1, 2, 3]), rkv, r.choice([4, 7, 16, 32, 40]), r.choice([4, 6, 16, 32, 40]), r.choice([1, 2, 3, 4, 6]))
+        owners.append(i)
+        layers.append(_layer(left, right, r.choice([0.3, 0.6, 1.0]), r.choice([0.3, 0.5, 1.0]), r.choice([None, 24, 50, 64])))
+    config = {"architecture": "Vugelix", "norm": {"eps": r.choice([1e-6, 1e-5, 1e-3])}, "vocab": r.choice([33, 64, 90, 131]),
+              "width": width, "embedding": {"scale": r.choice([1.0, 4.0, 10.0])}, "logit_scale": r.choice([0.25, 1.0, 2.0]),
+              "layers": layers}
+    streams = r.choice([None, 1, 2, 3, 4, 8])
+    if streams is not None:
+        config["streams"] = streams
+    return config

@@ -1,8 +1,10 @@
 // A feed-forward made of many small gated feed-forwards of which every token uses a few.
-//   nhv_route_topk        from a row's float router logits the ``top`` largest: their numbers and scores (sigmoid)
+//   nhv_route_topk        from a row's float router logits (plus an optional bias) the ``top`` largest: their numbers and
+//                         scores (the sigmoid of each, or the softmax over the chosen logits alone)
 //   nhv_experts_gate_up   for every (token, chosen expert): act(s G_e h) * (s U_e h), s the score: the expert's input is
 //                         s h, and a product is linear in its rows, so the score multiplies the finished float sums
-//   nhv_experts_down      out[t] = sum over the token's experts of D_e u[t, j]
+//                         (no scores: s = 1, for a design whose scores weigh the experts' outputs)
+//   nhv_experts_down      out[t] = sum over the token's experts of [w[t, j]] D_e u[t, j] [+ one more row added to all]
 // One wave per output: a sum runs over its inner index in an order that depends on the sizes only, so a row's result
 // does not depend on its batch. Weights of all experts lie in one tensor, [experts, 2 ff, width] (gate rows, then up
 // rows) and [experts, width, ff].
@@ -10,14 +12,15 @@
 #include <math.h>
 
 // z [T, E] float logits. One wave per token: the ``top`` largest in turn, the lower number among equals.
-__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids,
-                                                         float* __restrict__ scores, int T, int E, int top) {
+__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
+                                                         int* __restrict__ ids, float* __restrict__ scores, int T, int E,
+                                                         int top, int mode) {
   extern __shared__ float z_all[];           // 4 waves x E logits
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
   float* z = z_all + (size_t)wave * E;
-  for (int e = lane; e < E; e += NHV_WAVE) z[e] = logits[(size_t)t * E + e];
+  for (int e = lane; e < E; e += NHV_WAVE) z[e] = logits[(size_t)t * E + e] + (bias ? bias[e] : 0.f);
   __builtin_amdgcn_wave_barrier();
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
@@ -35,17 +38,30 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
     if (at == 0x7fffffff) at = 0;            // (every logit is no number: the first expert)
     if (lane == 0) {
       ids[(size_t)t * top + j] = at;
-      scores[(size_t)t * top + j] = 1.0f / (1.0f + expf(-best));
+      scores[(size_t)t * top + j] = mode == 0 ? 1.0f / (1.0f + expf(-best)) : best;
       z[at] = -INFINITY;                     // a chosen expert is out of the next rounds
     }
     __builtin_amdgcn_wave_barrier();
   }
+  if (mode == 1 && lane == 0) {              // the softmax over the chosen logits alone; the first is the largest
+    float* s = scores + (size_t)t * top;
+    const float m = s[0];
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) {
+      s[j] = expf(s[j] - m);
+      sum += s[j];
+    }
+    for (int j = 0; j < top; ++j) s[j] /= sum;
+  }
 }
 
-extern "C" int nhv_route_topk(const void* logits, void* ids, void* scores, int T, int E, int top, void* stream) {
+// mode 0: a score is the sigmoid of its logit; 1: the scores are the softmax over the chosen logits
+extern "C" int nhv_route_topk(const void* logits, const void* bias, void* ids, void* scores, int T, int E, int top, int mode,
+                              void* stream) {
   NHV_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E && E <= 4096, "route_topk: bad sizes T=%d E=%d (up to 4096) top=%d", T, E, top);
+  NHV_REQUIRE(mode == 0 || mode == 1, "route_topk: mode %d", mode);
   hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), 4 * (size_t)E * sizeof(float), (hipStream_t)stream,
-                     (const float*)logits, (int*)ids, (float*)scores, T, E, top);
+                     (const float*)logits, (const float*)bias, (int*)ids, (float*)scores, T, E, top, mode);
   NHV_LAUNCH_CHECK("route_topk");
   return 0;
 }
@@ -112,7 +128,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
   sg = wave_sum(sg);
   su = wave_sum(su);
   if (lane == 0) {
-    const float s = scores[pair];
+    const float s = scores ? scores[pair] : 1.0f;
     u[(size_t)pair * F + f] = from_f32<T>(nhv_expert_act(s * sg, act) * (s * su));
   }
 }
@@ -135,11 +151,12 @@ extern "C" int nhv_experts_gate_up(const void* h, const void* ids, const void* s
   return 0;
 }
 
-// out[t, n] = sum over j < top (rising), each a sum over f: one wave per n.
+// out[t, n] = sum over j < top (rising), each a sum over f [times weights[t, j]], [plus add[t, n]]: one wave per n.
 template <typename T>
 __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__ u, const int* __restrict__ ids,
                                                            const T* __restrict__ down, T* __restrict__ out, int W, int F,
-                                                           int top, int E) {
+                                                           int top, int E, const float* __restrict__ weights,
+                                                           const T* __restrict__ add) {
   const int t = blockIdx.x;
   const int n = blockIdx.y * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -162,23 +179,23 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
     } else {
       for (int f = lane; f < F; f += NHV_WAVE) s = fmaf(to_f32(d[f]), to_f32(x[f]), s);
     }
-    total += wave_sum(s);
+    total += weights ? weights[(size_t)t * top + j] * wave_sum(s) : wave_sum(s);
   }
-  if (lane == 0) out[(size_t)t * W + n] = from_f32<T>(total);
+  if (lane == 0) out[(size_t)t * W + n] = from_f32<T>(add ? total + to_f32(add[(size_t)t * W + n]) : total);
 }
 
 extern "C" int nhv_experts_down(const void* u, const void* ids, const void* down, void* out, int T, int W, int F, int top,
-                                int E, int dtype, void* stream) {
+                                int E, const void* weights, const void* add, int dtype, void* stream) {
   NHV_REQUIRE(T > 0 && W > 0 && F > 0 && top > 0 && E > 0, "experts_down: bad sizes T=%d W=%d F=%d top=%d E=%d", T, W, F, top, E);
   NHV_REQUIRE((W + 3) / 4 <= 65535, "experts_down: width %d is beyond this kernel's grid", W);
   const dim3 grid(T, (W + 3) / 4);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == NHV_F32)
     hipLaunchKernelGGL(experts_down_kernel<float>, grid, dim3(256), 0, s, (const float*)u, (const int*)ids,
-                       (const float*)down, (float*)out, W, F, top, E);
+                       (const float*)down, (float*)out, W, F, top, E, (const float*)weights, (const float*)add);
   else if (dtype == NHV_BF16)
     hipLaunchKernelGGL(experts_down_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)u, (const int*)ids,
-                       (const bf16_t*)down, (bf16_t*)out, W, F, top, E);
+                       (const bf16_t*)down, (bf16_t*)out, W, F, top, E, (const float*)weights, (const bf16_t*)add);
   else
     return nhv_fail("experts_down: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("experts_down");
@@ -314,7 +331,7 @@ __global__ __launch_bounds__(64 * WAVES) void experts_grouped_kernel(const bf16_
   }
   // wave ``mt`` adds the waves' partial sums of tile (nt, mt) in the order of the waves and writes that tile
   const int my_pair = wave < MT ? places[wave * 16 + col] : -1;
-  const float s = (GLU && my_pair >= 0) ? scores[my_pair] : 1.0f;
+  const float s = (GLU && scores && my_pair >= 0) ? scores[my_pair] : 1.0f;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     float v[NA][4];
@@ -440,7 +457,7 @@ __global__ __launch_bounds__(64 * WM * WN) void experts_tiled_kernel(const bf16_
   for (int mt = 0; mt < MT; ++mt) {
     const int pair = places[(wm * MT + mt) * 16 + col];
     if (pair < 0) continue;
-    const float s = GLU ? scores[pair] : 1.0f;
+    const float s = (GLU && scores) ? scores[pair] : 1.0f;
 #pragma unroll
     for (int a = 0; a < NH; ++a)
 #pragma unroll
@@ -503,22 +520,24 @@ extern "C" int nhv_experts_grouped_down(const void* u, const void* down, void* y
   return 0;
 }
 
-// out[t, n] = sum over j < top (rising) of y[t * top + j, n]
-__global__ void experts_combine_kernel(const float* __restrict__ y, bf16_t* __restrict__ out, int W, int top, size_t total) {
+// out[t, n] = sum over j < top (rising) of [weights[t, j]] y[t * top + j, n], [plus add[t, n]]
+__global__ void experts_combine_kernel(const float* __restrict__ y, bf16_t* __restrict__ out, int W, int top, size_t total,
+                                       const float* __restrict__ weights, const bf16_t* __restrict__ add) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
     const size_t t = i / W, n = i % W;
     float sum = 0.f;
-    for (int j = 0; j < top; ++j) sum += y[(t * top + j) * W + n];
-    out[i] = (bf16_t)sum;
+    for (int j = 0; j < top; ++j) sum += weights ? weights[t * top + j] * y[(t * top + j) * W + n] : y[(t * top + j) * W + n];
+    out[i] = (bf16_t)(add ? sum + (float)add[i] : sum);
   }
 }
 
-extern "C" int nhv_experts_combine(const void* y, void* out, int T, int W, int top, void* stream) {
+extern "C" int nhv_experts_combine(const void* y, void* out, int T, int W, int top, const void* weights, const void* add,
+                                   void* stream) {
   NHV_REQUIRE(T > 0 && W > 0 && top > 0, "experts_combine: bad sizes T=%d W=%d top=%d", T, W, top);
   const size_t total = (size_t)T * W;
   const int blocks = (int)((total + 255) / 256 > 65535 * 4 ? 65535 * 4 : (total + 255) / 256);
   hipLaunchKernelGGL(experts_combine_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const float*)y, (bf16_t*)out,
-                     W, top, total);
+                     W, top, total, (const float*)weights, (const bf16_t*)add);
   NHV_LAUNCH_CHECK("experts_combine");
   return 0;
 }

@@ -144,73 +144,103 @@ extern "C" int nhv_depth_mix(const void* x, const void* a, const void* b, void* 
   return 0;
 }
 
-// ---------------------------------------------------------------- split, bias, rotation, cache write
-// One wave per (token, head of q | k | v). qkv: [T, Hq D + Hkv D + Hkv E] (with_kv) or [T, Hq D]. qk_freqs [rot / 2]:
-// pair (i, i + rot / 2) of a query or key head at position p turns by p * qk_freqs[i]; the coordinates from rot on
-// pass. v_freqs [E / 2] or null: pair (m, m + E / 2) of a value head turns by p * v_freqs[m].
+// ---------------------------------------------------------------- split, bias, rotation, store
+// qkv [T, ld]: q (Hq heads of D) | k (Hkv heads of D) | v (Hv heads of E) | further columns of another reader; one wave
+// per (token, head). A query or key head at position p turns over its first ``rot`` coordinates by p * qk_freqs[i]:
+// pair (i, i + rot / 2), or (2i, 2i + 1) where ``interleaved``; the coordinates from rot on pass. v_freqs [E / 2] or
+// null: pair (m, m + E / 2) of a value head turns by p * v_freqs[m]. ``unit``: after the rotation every query and key
+// head is divided by its root mean square (unit_eps under the root), in float before anything is rounded.
+// ``v_from_k``: there are no value columns; value head g is key head g as projected (bias added, not turned, not
+// normed). ``maps`` n > 1: query and key heads lie in the projection as [head][map] and are written as
+// [map][head] (map c of head s / n goes to head c * heads / n + s / n), so that map c's query heads meet map c's key
+// heads under the ordinary grouping of heads; the Hkv / n value heads are stored once for every map.
 template <typename T>
 __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
                                           const float* __restrict__ qk_freqs, int rot, const float* __restrict__ v_freqs,
                                           const int* __restrict__ positions, const int* __restrict__ slot_mapping,
                                           T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq,
-                                          int Hkv, int D, int E, int heads, int ld) {
+                                          int Hkv, int Hv, int D, int E, int heads, int ld, int interleaved, int unit,
+                                          float unit_eps, int v_from_k, int maps) {
+  extern __shared__ float staged[];            // max(D, E) floats: the head after bias and rotation
   const int t = blockIdx.x / heads, head = blockIdx.x % heads;
   const float p = (float)positions[t];
-  int col, size, half;
+  int col, size, half, copies = 1, copy_stride = 0;
+  bool normed = false, pairs_adjacent = false;
   const float* freqs;
   T* dst;
   if (head < Hq) {
-    col = head * D; size = D; half = rot / 2; freqs = qk_freqs;
-    dst = q_out + ((size_t)t * Hq + head) * D;
+    col = head * D; size = D; half = rot / 2; freqs = qk_freqs; normed = unit; pairs_adjacent = interleaved;
+    const int to = (head % maps) * (Hq / maps) + head / maps;
+    dst = q_out + ((size_t)t * Hq + to) * D;
   } else {
     const int slot = slot_mapping[t];
     if (slot < 0) return;                      // a row that stores nothing (padding of a recorded step)
     if (head < Hq + Hkv) {
       const int g = head - Hq;
-      col = Hq * D + g * D; size = D; half = rot / 2; freqs = qk_freqs;
-      dst = k_cache + ((size_t)slot * Hkv + g) * D;
+      col = Hq * D + g * D; size = D; half = rot / 2; freqs = qk_freqs; normed = unit; pairs_adjacent = interleaved;
+      const int to = (g % maps) * (Hkv / maps) + g / maps;
+      dst = k_cache + ((size_t)slot * Hkv + to) * D;
     } else {
       const int g = head - Hq - Hkv;
-      col = (Hq + Hkv) * D + g * E; size = E; half = v_freqs ? E / 2 : 0; freqs = v_freqs;
+      col = v_from_k ? Hq * D + g * D : (Hq + Hkv) * D + g * E;
+      size = E; half = v_freqs ? E / 2 : 0; freqs = v_freqs;
       dst = v_cache + ((size_t)slot * Hkv + g) * E;
+      copies = maps; copy_stride = Hv * E;
     }
   }
   const T* src = qkv + (size_t)t * ld + col;
   const T* bs = bias ? bias + col : nullptr;
   // the bias joins a projection that was rounded to the rows' type, and the sum is rounded again (the product's own result)
   auto value = [&](int i) { return bs ? to_f32(from_f32<T>(to_f32(src[i]) + to_f32(bs[i]))) : to_f32(src[i]); };
+  float ss = 0.f;
   for (int i = threadIdx.x; i < size - half; i += blockDim.x) {
     if (i < half) {
-      const float u = value(i), v = value(i + half);
+      const int a = pairs_adjacent ? 2 * i : i, b = pairs_adjacent ? 2 * i + 1 : i + half;
+      const float u = value(a), v = value(b);
       float sn, cs;
       sincosf(p * freqs[i], &sn, &cs);
-      dst[i] = from_f32<T>(u * cs - v * sn);
-      dst[i + half] = from_f32<T>(v * cs + u * sn);
+      const float x = u * cs - v * sn, y = v * cs + u * sn;
+      staged[a] = x;
+      staged[b] = y;
+      ss = fmaf(x, x, fmaf(y, y, ss));
     } else {
-      dst[i + half] = from_f32<T>(value(i + half));
+      const float x = value(i + half);
+      staged[i + half] = x;
+      ss = fmaf(x, x, ss);
     }
   }
+  const float r = normed ? 1.0f / sqrtf(wave_sum(ss) / (float)size + unit_eps) : 1.0f;
+  __syncthreads();
+  for (int c = 0; c < copies; ++c)
+    for (int i = threadIdx.x; i < size; i += blockDim.x) dst[(size_t)c * copy_stride + i] = from_f32<T>(staged[i] * r);
 }
 
 extern "C" int nhv_rotary_split_write(const void* qkv, const void* bias, const void* qk_freqs, int rot, const void* v_freqs,
                                       const void* positions, const void* slot_mapping, void* q_out, void* k_cache,
                                       void* v_cache, int T, int Hq, int Hkv, int D, int E, int with_kv, int more_columns,
-                                      int dtype, void* stream) {
+                                      int interleaved, int unit, float unit_eps, int v_from_k, int maps, int dtype,
+                                      void* stream) {
   NHV_REQUIRE(more_columns >= 0, "rotary_split_write: %d columns after the projection", more_columns);
   NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && D > 0 && E > 0, "rotary_split_write: bad sizes T=%d Hq=%d Hkv=%d D=%d E=%d", T, Hq, Hkv, D, E);
   NHV_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "rotary_split_write: rotary size %d with head size %d", rot, D);
   NHV_REQUIRE(rot == 0 || qk_freqs, "rotary_split_write: a rotary size without frequencies");
   NHV_REQUIRE(!v_freqs || E % 2 == 0, "rotary_split_write: value heads of odd size %d cannot be turned", E);
   NHV_REQUIRE(!with_kv || (slot_mapping && k_cache && v_cache), "rotary_split_write: cache write without cache");
-  const int heads = with_kv ? Hq + 2 * Hkv : Hq;
-  const int ld = (with_kv ? Hq * D + Hkv * (D + E) : Hq * D) + more_columns;   // (columns that belong to another reader)
+  NHV_REQUIRE(maps >= 1 && Hq % maps == 0 && Hkv % maps == 0, "rotary_split_write: %d maps with %d and %d heads", maps, Hq, Hkv);
+  NHV_REQUIRE(!v_from_k || (E == D && maps == 1), "rotary_split_write: values that are the keys as projected have the keys' size and one map");
+  NHV_REQUIRE(!unit || unit_eps >= 0.f, "rotary_split_write: eps %g", (double)unit_eps);
+  const int Hv = Hkv / maps;
+  const int heads = with_kv ? Hq + Hkv + Hv : Hq;
+  const int ld = (with_kv ? Hq * D + Hkv * D + (v_from_k ? 0 : Hv * E) : Hq * D) + more_columns;   // (columns that belong to another reader)
   NHV_REQUIRE((long long)T * heads < (1ll << 31), "rotary_split_write: too many tokens");
+  const size_t lds = (size_t)(D > E ? D : E) * sizeof(float);
+  NHV_REQUIRE(lds <= 64 * 1024, "rotary_split_write: heads of %d and %d entries are beyond this kernel", D, E);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(TT)                                                                                                   \
-  hipLaunchKernelGGL(rotary_split_write_kernel<TT>, dim3((unsigned)((size_t)T * heads)), dim3(NHV_WAVE), 0, s,       \
+  hipLaunchKernelGGL(rotary_split_write_kernel<TT>, dim3((unsigned)((size_t)T * heads)), dim3(NHV_WAVE), lds, s,     \
                      (const TT*)qkv, (const TT*)bias, (const float*)qk_freqs, rot, (const float*)v_freqs,            \
-                     (const int*)positions, (const int*)slot_mapping, (TT*)q_out, (TT*)k_cache, (TT*)v_cache, Hq, Hkv, D, \
-                     E, heads, ld)
+                     (const int*)positions, (const int*)slot_mapping, (TT*)q_out, (TT*)k_cache, (TT*)v_cache, Hq, Hkv, Hv, \
+                     D, E, heads, ld, interleaved, unit, unit_eps, v_from_k, maps)
   if (dtype == NHV_F32) LAUNCH(float);
   else if (dtype == NHV_BF16) LAUNCH(bf16_t);
   else return nhv_fail("rotary_split_write: unknown dtype %d", dtype);

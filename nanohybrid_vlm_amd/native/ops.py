@@ -20,7 +20,7 @@ from . import library
 
 CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "gemm_fewrows_bf16.hip", "attention_generic.hip",
                 "sampling.hip", "measure.hip", "stream_mixing.hip", "delta_rule.hip", "parallel_block.hip", "latent_attention.hip",
-                "routed_experts.hip", "hyper_streams.hip"]
+                "routed_experts.hip", "hyper_streams.hip", "head_outputs.hip", "sandwich_norms.hip"]
 BLAS_SOURCES = ["error.hip", "gemm_library.hip"]                                                   # the vendor's matrix library, algorithm by number
 BLAS_LINK = ["-lhipblaslt"]
 ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefill_bf16.hip"]      # compiled once per head size
@@ -237,10 +237,28 @@ class NativeBackend:
                    _ptr(wb), ctypes.c_float(pair_eps), dtype_code(a), _stream())
 
     def rotary_split_write(self, qkv, bias, qk_freqs, rot, v_freqs, positions, slot_mapping, q_out, k_cache, v_cache,
-                           Hq, Hkv, D, E, with_kv, more_columns=0):
+                           Hq, Hkv, D, E, with_kv, more_columns=0, interleaved=False, unit_eps=None, values_from_keys=False,
+                           maps=1):
         self._call("nhv_rotary_split_write", _ptr(qkv), _ptr(bias), _ptr(qk_freqs), rot, _ptr(v_freqs), _ptr(positions),
                    _ptr(slot_mapping), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], Hq, Hkv, D, E,
-                   int(with_kv), more_columns, dtype_code(qkv), _stream())
+                   int(with_kv), more_columns, int(interleaved), int(unit_eps is not None), ctypes.c_float(unit_eps or 0.0),
+                   int(values_from_keys), maps, dtype_code(qkv), _stream())
+
+    # -- what heads' results pass before the output projection; a layer normed on both sides of its sublayers --
+    def differential_combine(self, a, lam, out, eps, post, gate=None):
+        T, H, E = out.shape
+        self._call("nhv_differential_combine", _ptr(a), _ptr(lam), _ptr(out), T, H, E, ctypes.c_float(eps),
+                   ctypes.c_float(post), *_gate_args(gate), dtype_code(a), _stream())
+
+    def gate_rows(self, x, gate):
+        T, N = x.shape
+        self._call("nhv_gate_rows", _ptr(x), *_gate_args(gate), T, N, dtype_code(x), _stream())
+
+    def sandwich_step(self, x, y, wb, eps_b, wa, eps_a, h):
+        T, W = x.shape
+        self._call("nhv_sandwich_step", _ptr(x), _ptr(y), dtype_code(y) if y is not None else 0, _ptr(wb),
+                   ctypes.c_float(eps_b), _ptr(wa), ctypes.c_float(eps_a), _ptr(h), dtype_code(h) if h is not None else 0,
+                   T, W, _stream())
 
     def turn_back(self, x, freqs, positions):
         T, H, E = x.shape
@@ -360,9 +378,9 @@ class NativeBackend:
                    ctypes.c_float(gain), _ptr(positions), T, H, dtype_code(src), _stream())
 
     # -- a feed-forward of many small experts --
-    def route_topk(self, logits, ids, scores):
+    def route_topk(self, logits, ids, scores, bias=None, mode=0):
         T, E = logits.shape
-        self._call("nhv_route_topk", _ptr(logits), _ptr(ids), _ptr(scores), T, E, ids.shape[1], _stream())
+        self._call("nhv_route_topk", _ptr(logits), _ptr(bias), _ptr(ids), _ptr(scores), T, E, ids.shape[1], mode, _stream())
 
     def experts_gate_up(self, h, ids, scores, gate_up, u, act):
         T, W = h.shape
@@ -370,7 +388,7 @@ class NativeBackend:
         self._call("nhv_experts_gate_up", _ptr(h), _ptr(ids), _ptr(scores), _ptr(gate_up), _ptr(u), T, W, F2 // 2,
                    ids.shape[1], E, act, dtype_code(h), _stream())
 
-    def experts_grouped(self, h, ids, scores, gate_up, down, out, act):
+    def experts_grouped(self, h, ids, scores, gate_up, down, out, act, weights=None, add=None):
         """Many rows in bfloat16: the pairs sorted by expert, then both products on the matrix cores, then the sum over
         a token's experts."""
         T, W = h.shape
@@ -392,13 +410,13 @@ class NativeBackend:
         y = torch.empty((P, W), dtype=torch.float32, device=h.device)
         self._call("nhv_experts_grouped_down", _ptr(u), _ptr(down), _ptr(y), _ptr(sorted_pairs), _ptr(tile_expert), W, F, TM,
                    tiles, _stream())
-        self._call("nhv_experts_combine", _ptr(y), _ptr(out), T, W, top, _stream())
+        self._call("nhv_experts_combine", _ptr(y), _ptr(out), T, W, top, _ptr(weights), _ptr(add), _stream())
 
-    def experts_down(self, u, ids, down, out):
+    def experts_down(self, u, ids, down, out, weights=None, add=None):
         T, W = out.shape
         E, _, F = down.shape
         self._call("nhv_experts_down", _ptr(u), _ptr(ids), _ptr(down), _ptr(out), T, W, F, ids.shape[1], E,
-                   dtype_code(u), _stream())
+                   _ptr(weights), _ptr(add), dtype_code(u), _stream())
 
     def _decode_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window, more=()):
         """Single tokens in bfloat16: keys split over waves, then merged. ``more``: the arguments of a cap on the
@@ -638,10 +656,12 @@ class NativeBackend:
             if M <= self.few_rows or (M <= 64 and self.own_kernels_only):
                 return self._call("nhv_gemm_skinny_bf16", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
                                   dtype_code(out), _stream())
-            if out.dtype == torch.bfloat16 and bias is None and not self.own_kernels_only:
+            if out.dtype == torch.bfloat16 and not self.own_kernels_only:
                 # many rows: the library's matrix product (the reference's linears are library calls too,
-                # nanovllm/layers/linear.py:88,192)
+                # nanovllm/layers/linear.py:88,192); a bias joins the rounded rows in a kernel of its own
                 torch.mm(x, w.t(), out=out)
+                if bias is not None:
+                    self._call("nhv_add_bias_rows", _ptr(out), _ptr(bias), M, N, dtype_code(out), _stream())
                 return None
             if out.dtype == torch.float32 and bias is None and not self.own_kernels_only and _MM_GIVES_FLOAT32:
                 # the logits of many rows: the library's product with float sums and a float result (270 us for 64
@@ -1378,22 +1398,38 @@ def rotate_interleaved(src: torch.Tensor, s_off: int, dst: torch.Tensor, d_off: 
 
 
 # ------------------------------------------------------------------ a feed-forward of many small experts
-def route_topk(logits: torch.Tensor, top: int):
-    """(numbers [tokens, top] int32, scores [tokens, top] float32) of the ``top`` experts with the largest logits, the
-    largest first, the lower number among equals; a score is the sigmoid of its logit."""
+ROUTER_SCORES = {"sigmoid": 0, "softmax_of_chosen": 1}
+
+
+def route_topk(logits: torch.Tensor, top: int, bias: torch.Tensor | None = None, scoring: str = "sigmoid"):
+    """(numbers [tokens, top] int32, scores [tokens, top] float32) of the ``top`` experts with the largest logits
+    (``bias`` [experts] float32 is added to them first), the largest first, the lower number among equals. ``scoring``
+    "sigmoid": a score is the sigmoid of its logit; "softmax_of_chosen": the scores are the softmax over the chosen
+    logits alone."""
     _need(logits.dim() == 2, "route_topk: logits must be [tokens, experts]")
     _dense(logits, "route_topk: logits", dtype=torch.float32)
     _need(0 < top <= logits.shape[1], lambda: f"route_topk: {top} of {logits.shape[1]} experts")
+    _need(scoring in ROUTER_SCORES, lambda: f"route_topk: scoring {scoring!r} is not known ({sorted(ROUTER_SCORES)} are)")
     ids = torch.empty((logits.shape[0], top), dtype=torch.int32, device=logits.device)
     scores = torch.empty((logits.shape[0], top), dtype=torch.float32, device=logits.device)
-    backend().route_topk(logits, ids, scores)
+    more = {}
+    if bias is not None:
+        _float32(bias, "route_topk: bias", (logits.shape[1],))
+        more["bias"] = bias
+    if scoring != "sigmoid":
+        more["mode"] = ROUTER_SCORES[scoring]
+    if logits.shape[0]:
+        backend().route_topk(logits, ids, scores, **more)
     return ids, scores
 
 
 def routed_experts(h: torch.Tensor, ids: torch.Tensor, scores: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
-                   activation: str = "silu") -> torch.Tensor:
+                   activation: str = "silu", scores_on: str = "input", add: torch.Tensor | None = None) -> torch.Tensor:
     """sum over a token's experts e (``ids``) of D_e (act(G_e x) * (U_e x)), x = score * h: the score multiplies the
-    expert's input. ``gate_up`` [experts, 2 ff, width] (gate rows, then up rows), ``down`` [experts, width, ff]."""
+    expert's input (``scores_on`` "input"); or of score * D_e (act(G_e h) * (U_e h)): the score weighs the expert's
+    output ("output"). ``add`` [tokens, width]: one more row added to every token's sum before it is rounded (an expert
+    that all tokens use). ``gate_up`` [experts, 2 ff, width] (gate rows, then up rows), ``down`` [experts, width, ff]."""
+    _need(scores_on in ("input", "output"), lambda: f"routed_experts: scores on {scores_on!r}")
     _need(h.dim() == 2, "routed_experts: h must be [tokens, width]")
     T, W = h.shape
     _dense(h, "routed_experts: h")
@@ -1408,13 +1444,21 @@ def routed_experts(h: torch.Tensor, ids: torch.Tensor, scores: torch.Tensor, gat
     _dense(scores, "routed_experts: scores", tuple(ids.shape), torch.float32)
     out = torch.empty((T, W), dtype=h.dtype, device=h.device)
     b = backend()
+    first, more = scores, {}
+    if scores_on == "output":
+        first, more = None, {"weights": scores}
+    if add is not None:
+        _dense(add, "routed_experts: add", (T, W), h.dtype)
+        more["add"] = add
+    if not T:
+        return out
     if (h.dtype == torch.bfloat16 and T > getattr(b, "few_rows", 0) and W % 8 == 0 and F % 8 == 0 and E <= 4096
             and hasattr(b, "experts_grouped")):
-        b.experts_grouped(h, ids, scores, gate_up, down, out, ACTIVATIONS[activation])
+        b.experts_grouped(h, ids, first, gate_up, down, out, ACTIVATIONS[activation], **more)
         return out
     u = torch.empty((T * ids.shape[1], F), dtype=h.dtype, device=h.device)
-    b.experts_gate_up(h, ids, scores, gate_up, u, ACTIVATIONS[activation])
-    b.experts_down(u, ids, down, out)
+    b.experts_gate_up(h, ids, first, gate_up, u, ACTIVATIONS[activation])
+    b.experts_down(u, ids, down, out, **more)
     return out
 
 # ------------------------------------------------------------------ layers that are not the pre-norm kind
@@ -1503,14 +1547,35 @@ def depth_mix(x: torch.Tensor, a, b: torch.Tensor | None, results: torch.Tensor,
 def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: torch.Tensor | None,
                        v_freqs: torch.Tensor | None, positions: torch.Tensor, slot_mapping, k_cache, v_cache,
                        num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, with_kv: bool = True,
-                       more_columns: int = 0) -> torch.Tensor:
+                       more_columns: int = 0, interleaved: bool = False, unit_eps: float | None = None,
+                       values_from_keys: bool = False, maps: int = 1) -> torch.Tensor:
     """Splits the packed projection q | k | v (``with_kv``) or q alone (followed by ``more_columns`` columns that
     another reader takes), adds the bias, turns pair (i, i + r) of every
     query and key head by position * qk_freqs[i] (r = len(qk_freqs); the coordinates from 2 r on pass), turns the
     value heads the same way over all their coordinates if ``v_freqs`` is given, stores keys and values at the
-    step's slots and returns q as [tokens, heads, head_dim]. Angles are taken in float from the position: no table."""
+    step's slots and returns q as [tokens, heads, head_dim]. Angles are taken in float from the position: no table.
+    ``interleaved``: the pairs are (2i, 2i + 1). ``unit_eps``: after the rotation every query and key head is divided
+    by its root mean square (this eps under the root), in float. ``values_from_keys``: the projection holds no value
+    columns; value head g is key head g as projected (not turned, not normed). ``maps`` n > 1: ``num_heads`` and
+    ``num_kv_heads`` count n maps per head, which lie in the projection as [head][map] and are returned and stored as
+    [map][head]; the projection holds num_kv_heads / n value heads, each stored once for every map (the value cache
+    has ``num_kv_heads`` heads)."""
     T = qkv.shape[0]
-    width = num_heads * head_dim + (num_kv_heads * (head_dim + value_dim) if with_kv else 0)
+    _need(maps >= 1 and num_heads % maps == 0 and num_kv_heads % maps == 0,
+          lambda: f"rotary_split_write: {maps} maps with {num_heads} and {num_kv_heads} heads")
+    _need(not values_from_keys or (value_dim == head_dim and maps == 1),
+          "rotary_split_write: values that are the keys as projected have the keys' size (and one map)")
+    value_columns = 0 if values_from_keys else (num_kv_heads // maps) * value_dim
+    width = num_heads * head_dim + (num_kv_heads * head_dim + value_columns if with_kv else 0)
+    more = {}
+    if interleaved:
+        more["interleaved"] = True
+    if unit_eps is not None:
+        more["unit_eps"] = float(unit_eps)
+    if values_from_keys:
+        more["values_from_keys"] = True
+    if maps != 1:
+        more["maps"] = int(maps)
     _need(more_columns >= 0, "rotary_split_write: a negative number of further columns")
     _dense(qkv, "rotary_split_write: qkv", (T, width + more_columns))
     dtype_code(qkv)
@@ -1538,8 +1603,72 @@ def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: t
         backend().rotary_split_write(qkv, bias, qk_freqs, rot, v_freqs if with_kv else None, positions,
                                      slot_mapping if with_kv else None, q_out, k_cache if with_kv else None,
                                      v_cache if with_kv else None, num_heads, num_kv_heads, head_dim, value_dim, with_kv,
-                                     **({"more_columns": int(more_columns)} if more_columns else {}))
+                                     **({"more_columns": int(more_columns)} if more_columns else {}), **more)
     return q_out
+
+
+def differential_combine(a: torch.Tensor, lam: torch.Tensor, eps: float, post: float, gate: tuple | None = None) -> torch.Tensor:
+    """a [tokens, 2 heads, size] holds two softmax maps per head over the same values, map 1 of all heads first. Returns
+    [tokens, heads, size]: o = a1 - lam a2, divided by sqrt(mean(o^2) + eps) over the head's entries, times ``post``
+    and, with ``gate`` = (rows [tokens, columns] of a's element type, first column), times sigmoid(rows[t, column + h]).
+    ``lam``: one float32 number on the device."""
+    _need(a.dim() == 3 and a.shape[1] % 2 == 0, "differential_combine: a must be [tokens, 2 heads, size]")
+    _dense(a, "differential_combine: a")
+    dtype_code(a)
+    _float32(lam, "differential_combine: lambda", (1,))
+    T, H, E = a.shape[0], a.shape[1] // 2, a.shape[2]
+    out = torch.empty((T, H, E), dtype=a.dtype, device=a.device)
+    more = {}
+    if gate is not None:
+        rows, col = gate
+        _need(rows.dim() == 2 and rows.shape[0] == T and 0 <= col and col + H <= rows.shape[1],
+              lambda: f"differential_combine: gates {tuple(rows.shape)} for {H} heads from column {col}")
+        _dense(rows, "differential_combine: gates", dtype=a.dtype)
+        more["gate"] = (rows, int(col))
+    if T:
+        backend().differential_combine(a, lam, out, float(eps), float(post), **more)
+    return out
+
+
+def gate_rows_(x: torch.Tensor, gate: tuple) -> torch.Tensor:
+    """x [tokens, n] in place: x[t, i] *= sigmoid(rows[t, first column + i]) with ``gate`` = (rows [tokens, columns] of
+    x's element type, first column)."""
+    _need(x.dim() == 2, "gate_rows: x must be [tokens, n]")
+    _dense(x, "gate_rows: x")
+    dtype_code(x)
+    rows, col = gate
+    _need(rows.dim() == 2 and rows.shape[0] == x.shape[0] and 0 <= col and col + x.shape[1] <= rows.shape[1],
+          lambda: f"gate_rows: gates {tuple(rows.shape)} for rows {tuple(x.shape)} from column {col}")
+    _dense(rows, "gate_rows: gates", dtype=x.dtype)
+    if x.shape[0]:
+        backend().gate_rows(x, (rows, int(col)))
+    return x
+
+
+def sandwich_step(x: torch.Tensor, add: tuple | None = None, read: tuple | None = None, rows_dtype=None):
+    """One launch between two sublayers of a layer that norms on both sides. x [tokens, width] float32, the stream.
+    ``add`` = (y [tokens, width], weight [width] float32, eps): x += y / sqrt(mean(y^2) + eps) * weight, in place.
+    ``read`` = (weight [width] float32, eps): returns x / sqrt(mean(x^2) + eps) * weight (of the new x) as rows of
+    ``rows_dtype``; without it None is returned."""
+    _need(x.dim() == 2, "sandwich_step: x must be [tokens, width]")
+    T, W = x.shape
+    _float32(x, "sandwich_step: x", (T, W))
+    _need(add is not None or read is not None, "sandwich_step: nothing to add and nothing to read")
+    y = wb = wa = h = None
+    eps_a = eps_b = 0.0
+    if add is not None:
+        y, wb, eps_b = add
+        _dense(y, "sandwich_step: y", (T, W))
+        dtype_code(y)
+        _float32(wb, "sandwich_step: the weight of the result's norm", (W,))
+    if read is not None:
+        wa, eps_a = read
+        _float32(wa, "sandwich_step: the weight of the norm that is read through", (W,))
+        h = torch.empty((T, W), dtype=rows_dtype or torch.float32, device=x.device)
+        dtype_code(h)
+    if T:
+        backend().sandwich_step(x, y, wb, float(eps_b), wa, float(eps_a), h)
+    return h
 
 
 def turn_back_(x: torch.Tensor, freqs: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:

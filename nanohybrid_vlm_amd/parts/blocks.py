@@ -275,3 +275,64 @@ class StreamMixBlock(Part):
             raise ValueError("a block of several streams is followed by a block of its kind and its number of streams")
         _, total = ops.streams_step(X, T, W, n, dtype, update=(mix, out, y), collapse=True)
         return total, None
+
+
+@BLOCKS.register("sandwich_norms")
+class SandwichNormsBlock(Part):
+    """A layer whose sublayers are normed on both sides, on a float32 stream x:
+        x <- x + mixer_out_norm(mixer(mixer_norm(x)));   x <- x + feed_forward_out_norm(feed_forward(feed_forward_norm(x))).
+    The four norms are RMS norms with a weight vector (``stream_rmsnorm``: the block reads their weight and eps). The
+    stream is what the block takes and returns as ``hidden`` (no residual beside it). One kernel stands between two
+    sublayers: it norms the result of the one, adds it to the stream and norms the new stream for the next, also across
+    the border to the next block of this kind. The feed-forward may be absent (then the block has two norms)."""
+
+    norm_slots = ("mixer_norm", "mixer_out_norm", "feed_forward_norm", "feed_forward_out_norm")
+    norms_ahead = True            # the model tells the block which block follows (``next_norm`` is that block's ``norm``)
+
+    def __init__(self, mixer, feed_forward, mixer_norm, mixer_out_norm, feed_forward_norm, feed_forward_out_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.mixer_out_norm = mixer_norm, mixer_out_norm
+        self.feed_forward_norm, self.feed_forward_out_norm = feed_forward_norm, feed_forward_out_norm
+        self.row_dtype = None
+
+    @property
+    def norm(self):
+        """What the block before this one is shown as the norm that takes its result: this block itself (its first
+        norm is read in that block's last kernel)."""
+        return self
+
+    def children(self):
+        out = {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "mixer_out_norm": self.mixer_out_norm}
+        if self.feed_forward is not None:
+            out.update({"feed_forward_norm": self.feed_forward_norm, "feed_forward": self.feed_forward,
+                        "feed_forward_out_norm": self.feed_forward_out_norm})
+        return out
+
+    def first_read(self) -> tuple:
+        """What the kernel before this block's mixer reads through: (norm weight, eps)."""
+        return (self.mixer_norm.weight, self.mixer_norm.eps)
+
+    def forward(self, hidden, residual, step, cache, next_norm=None):
+        if residual is not None:
+            raise ValueError("this block carries its stream itself and takes no residual beside it")
+        if hidden.dtype != torch.float32:
+            hidden = hidden.float()
+        dtype = self.row_dtype or torch.float32
+        ahead = step.scratch.pop("sandwich_rows_ahead", None)
+        if ahead is not None and ahead[0] is self and ahead[1] is hidden:
+            h = ahead[2]                           # the block before has read this block's first input already
+        else:
+            h = ops.sandwich_step(hidden, read=self.first_read(), rows_dtype=dtype)
+        y = self.mixer.forward(h, step, cache)
+        pending = (y, self.mixer_out_norm.weight, self.mixer_out_norm.eps)
+        if self.feed_forward is not None:
+            h = ops.sandwich_step(hidden, add=pending, read=(self.feed_forward_norm.weight, self.feed_forward_norm.eps),
+                                  rows_dtype=dtype)
+            y = self.feed_forward.forward(h, step)
+            pending = (y, self.feed_forward_out_norm.weight, self.feed_forward_out_norm.eps)
+        if isinstance(next_norm, SandwichNormsBlock):
+            h = ops.sandwich_step(hidden, add=pending, read=next_norm.first_read(), rows_dtype=dtype)
+            step.scratch["sandwich_rows_ahead"] = (next_norm, hidden, h)
+        else:
+            ops.sandwich_step(hidden, add=pending)
+        return hidden, None

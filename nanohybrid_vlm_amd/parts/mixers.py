@@ -1,7 +1,8 @@
 """Token mixers. ``GQAAttention`` follows nanovllm/models/qwen3.py:14-88 and
 nanovllm/layers/attention.py:43-75. ``RotaryAttention`` is softmax attention in a more general make (value heads of
 their own size, biases, a chunk mask, turned values, keys and values lent by another layer), ``GatedDeltaRule`` a
-recurrent mixer with a matrix of state per head, ``NormedPair`` two mixers side by side."""
+recurrent mixer with a matrix of state per head, ``NormedPair`` two mixers side by side, ``DifferentialAttention`` the
+difference of two softmax maps per head over the same values."""
 from __future__ import annotations
 
 import torch
@@ -95,11 +96,18 @@ class RotaryAttention(Part):
     borrows from (keys as stored, after rotation) with queries, mask and output projection of its own.
     ``softcap`` c: a score s (after the scale) becomes c tanh(s / c). ``sink`` z: the softmax's denominator holds one
     more term exp(z), a key of that score that has no value. ``head_gate``: head h's result is multiplied by
-    sigmoid(w_h . x), x the mixer's input; the rows w_h are the last ``num_heads`` rows of the packed projection."""
+    sigmoid(w_h . x), x the mixer's input; the rows w_h are the last ``num_heads`` rows of the packed projection.
+    ``element_gate``: the concatenated heads are multiplied entry by entry with sigmoid(G x); the rows of G are the
+    last ``num_heads * value_dim`` rows of the packed projection. ``rotation``: which coordinates make a pair,
+    "halves" (i, i + r / 2) or "interleaved" (2i, 2i + 1). ``unit_norm_eps``: after the rotation every query and key head
+    is divided by its root mean square (this eps under the root). ``values_are_keys``: there is no value projection; a
+    token's values are its keys as projected, before rotation and norm (``value_dim`` equals ``head_dim``)."""
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
                  bias: bool, position, chunk: int | None = None, window: int | None = None, rotate_values: bool = False,
-                 own_kv: bool = True, softcap: float | None = None, sink: float | None = None, head_gate: bool = False):
+                 own_kv: bool = True, softcap: float | None = None, sink: float | None = None, head_gate: bool = False,
+                 element_gate: bool = False, rotation: str = "halves", unit_norm_eps: float | None = None,
+                 values_are_keys: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} key/value heads")
         if window and chunk:
@@ -114,17 +122,30 @@ class RotaryAttention(Part):
             raise ValueError(f"a cap on the scores must be positive, got {softcap}")
         if head_gate and bias:
             raise ValueError("a gate per head and biases are not taken together")
+        if element_gate and (head_gate or bias):
+            raise ValueError("a gate per entry is not taken together with a gate per head or with biases")
+        if rotation not in ("halves", "interleaved"):
+            raise ValueError(f"rotation {rotation!r} is not known ('halves' and 'interleaved' are)")
+        if unit_norm_eps is not None and not unit_norm_eps >= 0:
+            raise ValueError(f"the eps of the unit norm must not be negative, got {unit_norm_eps}")
+        if values_are_keys and (value_dim != head_dim or rotate_values or not own_kv):
+            raise ValueError("values that are the keys as projected have the keys' size, are not turned and are the layer's own")
         self.softcap, self.sink, self.head_gate = softcap, sink, bool(head_gate)
+        self.element_gate, self.rotation, self.unit_norm_eps = bool(element_gate), rotation, unit_norm_eps
+        self.values_are_keys = bool(values_are_keys)
         self.qkv_weight = self.qkv_bias = self.o_weight = None
 
     def _packed_width(self) -> int:
         width = self.num_heads * self.head_dim
         if self.own_kv:
-            width += self.num_kv_heads * (self.head_dim + self.value_dim)
+            width += self.num_kv_heads * (self.head_dim + (0 if self.values_are_keys else self.value_dim))
         return width
 
+    def _gate_columns(self) -> int:
+        return self.num_heads if self.head_gate else (self.num_heads * self.value_dim if self.element_gate else 0)
+
     def param_specs(self):
-        gates = self.num_heads if self.head_gate else 0
+        gates = self._gate_columns()
         specs = {"qkv.weight": ParamSpec((self._packed_width() + gates, self.hidden_size)),
                  "o.weight": ParamSpec((self.hidden_size, self.num_heads * self.value_dim))}
         if self.bias:
@@ -145,10 +166,10 @@ class RotaryAttention(Part):
         if not self.own_kv and cache.writes:
             raise ValueError("an attention layer without key and value projections must borrow another entry's cache")
         qkv = ops.linear(x, self.qkv_weight)
-        gates = self.num_heads if self.head_gate else 0
+        gates = self._gate_columns()
         if self.own_kv and not writes:               # a layer with projections of its own that reads a lent cache
             if gates:
-                raise ValueError("a layer with a gate per head and projections of its own cannot read a lent cache")
+                raise ValueError("a layer with gates and projections of its own cannot read a lent cache")
             qkv = qkv[:, :self.num_heads * self.head_dim].contiguous()
         bias = self.qkv_bias if (self.qkv_bias is None or writes or not self.own_kv) else \
             self.qkv_bias[:self.num_heads * self.head_dim].contiguous()
@@ -156,14 +177,94 @@ class RotaryAttention(Part):
         v_freqs = self.position.frequencies_for(self.value_dim) if self.rotate_values else None
         q = ops.rotary_split_write(qkv, bias, freqs, v_freqs, step.token_positions, tables.slot_mapping, cache.k, cache.v,
                                    self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, with_kv=writes,
-                                   more_columns=gates)
+                                   more_columns=gates, interleaved=self.rotation == "interleaved",
+                                   unit_eps=self.unit_norm_eps, values_from_keys=self.values_are_keys)
         # (the gates stay where the projection left them: the attention kernels read them from the packed rows)
         o = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window, self.chunk,
                                 softcap=self.softcap, sink=self.sink,
-                                gate=(qkv, qkv.shape[1] - gates) if gates else None)
+                                gate=(qkv, qkv.shape[1] - gates) if self.head_gate else None)
         if self.rotate_values:
             ops.turn_back_(o, v_freqs, step.token_positions)
-        return ops.linear(o.view(o.shape[0], self.num_heads * self.value_dim), self.o_weight)
+        o = o.view(o.shape[0], self.num_heads * self.value_dim)
+        if self.element_gate:
+            ops.gate_rows_(o, (qkv, qkv.shape[1] - gates))
+        return ops.linear(o, self.o_weight)
+
+
+@MIXERS.register("differential_attention")
+class DifferentialAttention(Part):
+    """Softmax attention whose heads each hold two maps: queries and keys have two parts per head ([map 1 | map 2], each
+    of ``head_dim`` entries, each turned by the position on its own), both maps read the same values
+    (``num_kv_heads`` heads of ``value_dim``), and head h's result is
+        o = a1 - lam a2,   lam = exp(lq1 . lk1) - exp(lq2 . lk2) + diff   (one number for the layer),
+    divided by its root mean square over the head's entries (``eps`` under the root, no weight), times (1 - diff) and,
+    with ``head_gate``, times sigmoid(w_h . x), x the mixer's input. Mask (``chunk`` or ``window``), grouping of heads,
+    scale and rotation (``position``: a ``rotary_frequencies`` encoding; ``rotation`` "halves" or "interleaved") are
+    those of ``RotaryAttention``; ``bias``: q, k, v and the output projection have biases.
+    To the cache and the attention kernels a map is a head: the step's queries go out as 2 ``num_heads`` heads, map 1
+    of all heads first, the keys as 2 ``num_kv_heads`` heads in the same order, so that the ordinary grouping of heads
+    pairs every map with its own keys; the values are stored once for every map."""
+
+    MAPS = 2
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
+                 diff: float, eps: float, bias: bool, position, chunk: int | None = None, window: int | None = None,
+                 rotation: str = "interleaved", head_gate: bool = False):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} key/value heads")
+        if window and chunk:
+            raise ValueError("a window or a chunk, not both")
+        if rotation not in ("halves", "interleaved"):
+            raise ValueError(f"rotation {rotation!r} is not known ('halves' and 'interleaved' are)")
+        if not eps >= 0:
+            raise ValueError(f"eps must not be negative, got {eps}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim, self.scale, self.diff, self.eps = head_dim, value_dim, scale, float(diff), eps
+        self.bias, self.position, self.chunk, self.window = bool(bias), position, chunk or None, window or None
+        self.rotation, self.head_gate = rotation, bool(head_gate)
+        self.lam = None
+
+    def _packed_width(self) -> int:
+        n = self.MAPS
+        return n * (self.num_heads + self.num_kv_heads) * self.head_dim + self.num_kv_heads * self.value_dim
+
+    def param_specs(self):
+        gates = self.num_heads if self.head_gate else 0
+        specs = {"qkv.weight": ParamSpec((self._packed_width() + gates, self.hidden_size)),
+                 "o.weight": ParamSpec((self.hidden_size, self.num_heads * self.value_dim))}
+        if self.bias:
+            specs["qkv.bias"] = ParamSpec((self._packed_width(),), init="zeros")
+            specs["o.bias"] = ParamSpec((self.hidden_size,), init="zeros")
+        for name in ("lq1", "lk1", "lq2", "lk2"):
+            specs[name] = ParamSpec((self.head_dim,), always_float32=True, init_mean=0.0, init_std=0.3)
+        return specs
+
+    def bind(self, params):
+        self.qkv_weight, self.o_weight = params["qkv.weight"], params["o.weight"]
+        self.qkv_bias, self.o_bias = params.get("qkv.bias"), params.get("o.bias")
+        # the layer's one number, from float32 parameters in float32, once
+        lam = torch.exp((params["lq1"] * params["lk1"]).sum()) - torch.exp((params["lq2"] * params["lk2"]).sum()) + self.diff
+        self.lam = lam.to(torch.float32).reshape(1).contiguous()
+
+    def cache_need(self):
+        return PagedKVNeed(self.MAPS * self.num_kv_heads, self.head_dim, self.window,
+                           None if self.value_dim == self.head_dim else self.value_dim, self.chunk)
+
+    def forward(self, x, step, cache: CacheView):
+        if not cache.writes:
+            raise ValueError("a layer of two maps per head keeps its own keys and values")
+        tables = step.groups[cache.group]
+        n, H, G = self.MAPS, self.num_heads, self.num_kv_heads
+        qkv = ops.linear(x, self.qkv_weight)
+        gates = H if self.head_gate else 0
+        freqs = self.position.frequencies() if self.position is not None and self.position.rotary_dim else None
+        q = ops.rotary_split_write(qkv, self.qkv_bias, freqs, None, step.token_positions, tables.slot_mapping, cache.k, cache.v,
+                                   n * H, n * G, self.head_dim, self.value_dim, more_columns=gates,
+                                   interleaved=self.rotation == "interleaved", maps=n)
+        a = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window, self.chunk)
+        o = ops.differential_combine(a, self.lam, self.eps, 1.0 - self.diff,
+                                     gate=(qkv, qkv.shape[1] - gates) if gates else None)
+        return ops.linear(o.view(o.shape[0], H * self.value_dim), self.o_weight, self.o_bias)
 
 
 @MIXERS.register("gated_delta_rule")

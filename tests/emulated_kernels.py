@@ -224,26 +224,32 @@ class EmulatedBackend:
         dst[:, :, d_off:d_off + rot] = self._turn_pairs(src[:, :, s_off:s_off + rot].float(), positions, freqs, gain).to(dst.dtype)
 
     # -- a feed-forward of many small experts
-    def route_topk(self, logits, ids, scores):
+    def route_topk(self, logits, ids, scores, bias=None, mode=0):
+        if bias is not None:
+            logits = logits + bias
         order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :ids.shape[1]]
         ids.copy_(order.to(torch.int32))
-        scores.copy_(torch.sigmoid(torch.gather(logits, 1, order)))
+        chosen = torch.gather(logits, 1, order)
+        scores.copy_(torch.sigmoid(chosen) if mode == 0 else torch.softmax(chosen, dim=-1))
 
     def experts_gate_up(self, h, ids, scores, gate_up, u, act):
         T, top = ids.shape
         F = gate_up.shape[1] // 2
         for t in range(T):
             for j in range(top):
-                e, s = int(ids[t, j]), scores[t, j]
+                e, s = int(ids[t, j]), (scores[t, j] if scores is not None else 1.0)
                 gu = gate_up[e].float() @ h[t].float()
                 u[t * top + j] = (self._act(s * gu[:F], act) * (s * gu[F:])).to(u.dtype)
 
-    def experts_down(self, u, ids, down, out):
+    def experts_down(self, u, ids, down, out, weights=None, add=None):
         T, top = ids.shape
         for t in range(T):
             total = torch.zeros(out.shape[1])
             for j in range(top):
-                total = total + down[int(ids[t, j])].float() @ u[t * top + j].float()
+                one = down[int(ids[t, j])].float() @ u[t * top + j].float()
+                total = total + (one if weights is None else weights[t, j] * one)
+            if add is not None:
+                total = total + add[t].float()
             out[t] = total.to(out.dtype)
 
     @staticmethod
@@ -255,26 +261,64 @@ class EmulatedBackend:
         return torch.cat((u * cos - v * sin, v * cos + u * sin, t[..., 2 * half:]), dim=-1)
 
     def rotary_split_write(self, qkv, bias, qk_freqs, rot, v_freqs, positions, slot_mapping, q_out, k_cache, v_cache,
-                           Hq, Hkv, D, E, with_kv, more_columns=0):
+                           Hq, Hkv, D, E, with_kv, more_columns=0, interleaved=False, unit_eps=None, values_from_keys=False,
+                           maps=1):
         T, dt = qkv.shape[0], qkv.dtype
         x = qkv.float()
         if more_columns:
             x = x[:, :x.shape[1] - more_columns]
         if bias is not None:
             x = (x + bias.float()).to(dt).float()
-        q = x[:, :Hq * D].reshape(T, Hq, D)
-        q_out.copy_((self._turned(q, positions, qk_freqs) if rot else q).to(dt))
+
+        def prepared(t):
+            """[T, heads, D] as projected -> turned, made unit vectors, the maps of all heads gathered map by map"""
+            if rot and interleaved:
+                ang = positions.float()[:, None] * qk_freqs[None, :]
+                cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+                u, w = t[..., 0:rot:2], t[..., 1:rot:2]
+                turned = torch.stack((u * cos - w * sin, w * cos + u * sin), dim=-1).flatten(-2)
+                t = torch.cat((turned, t[..., rot:]), dim=-1)
+            elif rot:
+                t = self._turned(t, positions, qk_freqs)
+            if unit_eps is not None:
+                t = t / torch.sqrt((t * t).mean(-1, keepdim=True) + unit_eps)
+            if maps > 1:
+                t = t.reshape(T, t.shape[1] // maps, maps, D).transpose(1, 2).reshape(T, -1, D)
+            return t
+
+        q_out.copy_(prepared(x[:, :Hq * D].reshape(T, Hq, D)).to(dt))
         if with_kv:
-            k = x[:, Hq * D:(Hq + Hkv) * D].reshape(T, Hkv, D)
-            v = x[:, (Hq + Hkv) * D:].reshape(T, Hkv, E)
-            if rot:
-                k = self._turned(k, positions, qk_freqs)
+            raw_k = x[:, Hq * D:(Hq + Hkv) * D].reshape(T, Hkv, D)
+            k = prepared(raw_k)
+            if values_from_keys:
+                v = raw_k
+            else:
+                v = x[:, (Hq + Hkv) * D:].reshape(T, Hkv // maps, E).repeat(1, maps, 1)
             if v_freqs is not None:
                 v = self._turned(v, positions, v_freqs)
             ok = slot_mapping >= 0
             slots = slot_mapping[ok].long()
             k_cache.view(-1, Hkv, D)[slots] = k[ok].to(dt)
             v_cache.view(-1, Hkv, E)[slots] = v[ok].to(dt)
+
+    def differential_combine(self, a, lam, out, eps, post, gate=None):
+        T, H, E = out.shape
+        a = a.float()
+        o = a[:, :H] - lam.float() * a[:, H:]
+        o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * post
+        if gate is not None:
+            o = o * torch.sigmoid(gate[0][:, gate[1]:gate[1] + H].float())[:, :, None]
+        out.copy_(o.to(out.dtype))
+
+    def gate_rows(self, x, gate):
+        x.copy_((x.float() * torch.sigmoid(gate[0][:, gate[1]:gate[1] + x.shape[1]].float())).to(x.dtype))
+
+    def sandwich_step(self, x, y, wb, eps_b, wa, eps_a, h):
+        if y is not None:
+            yf = y.float()
+            x.add_(yf / torch.sqrt((yf * yf).mean(-1, keepdim=True) + eps_b) * wb)
+        if wa is not None:
+            h.copy_((x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps_a) * wa).to(h.dtype))
 
     def turn_back(self, x, freqs, positions):
         x.copy_(self._turned(x.float(), positions, freqs, sign=-1.0).to(x.dtype))

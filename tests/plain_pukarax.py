@@ -201,3 +201,12 @@ def forward(config: dict, tensors: dict, tokens, dtype=torch.float64, streams: l
         if streams is not None:
             streams.append(x.clone())
     return (rms_norm(x, W["final.norm"], eps) @ W["embed"].T) * config["logit_scale"]
+
+
+def greedy_generate(config: dict, tensors: dict, prompt, n: int, dtype=torch.float64) -> list[int]:
+    """The ``n`` tokens that follow ``prompt`` when the most likely token is taken each time (the whole sequence is
+    computed anew for every token)."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(config, tensors, toks, dtype)[-1].argmax()))
+    return toks[len(prompt):]

@@ -19,9 +19,10 @@ For these two ``value`` is generated tokens a second over the whole run, prompts
 ``--workload projections`` is a diagnosis, not the benchmark: a layer's matrix products alone, cold, beside a kernel
 that only reads the same bytes (see ``bench_projections``).
 
-``--workload design --shape pevazen-1b|pevazen-8b|fazovik-1b|fazovik-8b|vugelix-1b|vugelix-8b [--layers L]``: a model of the Pevazen, the
-Fazovik or the Vugelix design (see ``architectures/``) beside a Qwen3 model (for Vugelix: a Pevazen model of pairs of
-mixers) of the same width, heads, feed-forward size, vocabulary and number of layers: one prompt of ``--prompt-tokens`` in one step, decoding at
+``--workload design --shape pevazen-1b|pevazen-8b|fazovik-1b|fazovik-8b|vugelix-1b|vugelix-8b|pukarax-1b|pukarax-8b [--layers L]``: a model of
+the Pevazen, the Fazovik, the Vugelix or the Pukarax design (see ``architectures/``) beside a Qwen3 model (for Vugelix:
+a Pevazen model of pairs of mixers; for Pukarax: a Fazovik model, whose feed-forwards are dense and routed in turn as
+well) of the same width, heads, feed-forward size, experts, vocabulary and number of layers: one prompt of ``--prompt-tokens`` in one step, decoding at
 ``--batch`` requests, and the time of every own kernel in one eager step of each kind (see ``bench_design``).
 """
 import argparse
@@ -422,7 +423,7 @@ def bench_design(args):
     from nanohybrid_vlm_amd.engine.runner import StepEntry
     from nanohybrid_vlm_amd.native import ops
 
-    name = args.shape if args.shape.startswith(("pevazen", "fazovik", "vugelix")) else "pevazen-1b"
+    name = args.shape if args.shape.startswith(("pevazen", "fazovik", "vugelix", "pukarax")) else "pevazen-1b"
     design = name.split("-")[0]
     new = json.loads(json.dumps(named_shapes()[name]))
     layers = args.layers or min(8, len(new["layers"]))
@@ -441,6 +442,13 @@ def bench_design(args):
             right = dict(r, decay_rank=128, gate_rank=128)
             entries.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": layer["mlp"]})
         twin = {"architecture": "Pevazen", "layers": entries, "norm": {"eps": 1e-6}, "vocab": new["vocab"], "width": new["width"]}
+    elif design == "pukarax":
+        # the closest model the engine has is Fazovik: attention layers whose feed-forwards are dense and routed in turn,
+        # with as many experts of the same size and as many a token; its named shape of the same size has the same
+        # width, heads, inner sizes and vocabulary
+        beside = "fazovik"
+        twin = json.loads(json.dumps(named_shapes()[name.replace("pukarax", "fazovik")]))
+        twin["layers"] = twin["layers"][:layers]
     elif design == "fazovik":
         # the twin has as many heads, of the size of this design's value heads, a quarter as many key/value heads, and
         # the dense layers' inner size in every layer

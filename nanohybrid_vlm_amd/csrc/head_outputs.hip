@@ -8,15 +8,15 @@
 #include "nhv_common.h"
 #include <math.h>
 
-// a [T, 2 H, E] with map 1 of all heads first, then map 2 ([map][head]); lambda [1] float; gate: null, or the gates of
+// a [T, 2 H, E]: per head its map 1, then its map 2 ([head][map]); lambda [1] float; gate: null, or the gates of
 // token t at gate[t * gate_ld + h]. out [T, H, E]. One wave per (token, head).
 template <typename T>
 __global__ void differential_combine_kernel(const T* __restrict__ a, const float* __restrict__ lambda, T* __restrict__ out,
                                             int H, int E, float eps, float post, const T* __restrict__ gate,
                                             long long gate_ld) {
   const int t = blockIdx.x / H, h = blockIdx.x % H;
-  const T* a1 = a + ((size_t)t * 2 * H + h) * E;
-  const T* a2 = a1 + (size_t)H * E;
+  const T* a1 = a + ((size_t)t * H + h) * 2 * E;
+  const T* a2 = a1 + E;
   const float lam = lambda[0];
   float ss = 0.f;
   for (int i = threadIdx.x; i < E; i += blockDim.x) {

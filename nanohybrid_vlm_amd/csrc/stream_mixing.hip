@@ -151,9 +151,10 @@ extern "C" int nhv_depth_mix(const void* x, const void* a, const void* b, void* 
 // null: pair (m, m + E / 2) of a value head turns by p * v_freqs[m]. ``unit``: after the rotation every query and key
 // head is divided by its root mean square (unit_eps under the root), in float before anything is rounded.
 // ``v_from_k``: there are no value columns; value head g is key head g as projected (bias added, not turned, not
-// normed). ``maps`` n > 1: query and key heads lie in the projection as [head][map] and are written as
-// [map][head] (map c of head s / n goes to head c * heads / n + s / n), so that map c's query heads meet map c's key
-// heads under the ordinary grouping of heads; the Hkv / n value heads are stored once for every map.
+// normed). ``maps`` n > 1: every query and key head holds n maps of D entries, [map 1 | map 2 | ...], each turned (and
+// normed) on its own; Hq and Hkv count maps. The n maps of a key head are stored side by side as one key of n D entries
+// (there are Hkv / n key heads, and as many value heads); a query map goes out as a head of n D entries of its own
+// with zeros in the other maps' places, so that its product with the stored key is its product with its own map.
 template <typename T>
 __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
                                           const float* __restrict__ qk_freqs, int rot, const float* __restrict__ v_freqs,
@@ -164,28 +165,29 @@ __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __
   extern __shared__ float staged[];            // max(D, E) floats: the head after bias and rotation
   const int t = blockIdx.x / heads, head = blockIdx.x % heads;
   const float p = (float)positions[t];
-  int col, size, half, copies = 1, copy_stride = 0;
+  int col, size, half;
   bool normed = false, pairs_adjacent = false;
   const float* freqs;
   T* dst;
   if (head < Hq) {
     col = head * D; size = D; half = rot / 2; freqs = qk_freqs; normed = unit; pairs_adjacent = interleaved;
-    const int to = (head % maps) * (Hq / maps) + head / maps;
-    dst = q_out + ((size_t)t * Hq + to) * D;
+    T* whole = q_out + ((size_t)t * Hq + head) * maps * D;
+    dst = whole + (head % maps) * D;
+    if (maps > 1)                              // the other maps' places
+      for (int i = threadIdx.x; i < maps * D; i += blockDim.x)
+        if (i / D != head % maps) whole[i] = from_f32<T>(0.f);
   } else {
     const int slot = slot_mapping[t];
     if (slot < 0) return;                      // a row that stores nothing (padding of a recorded step)
     if (head < Hq + Hkv) {
       const int g = head - Hq;
       col = Hq * D + g * D; size = D; half = rot / 2; freqs = qk_freqs; normed = unit; pairs_adjacent = interleaved;
-      const int to = (g % maps) * (Hkv / maps) + g / maps;
-      dst = k_cache + ((size_t)slot * Hkv + to) * D;
+      dst = k_cache + ((size_t)slot * Hkv + g) * D;          // (map g % maps of key head g / maps: the same place)
     } else {
       const int g = head - Hq - Hkv;
       col = v_from_k ? Hq * D + g * D : (Hq + Hkv) * D + g * E;
       size = E; half = v_freqs ? E / 2 : 0; freqs = v_freqs;
-      dst = v_cache + ((size_t)slot * Hkv + g) * E;
-      copies = maps; copy_stride = Hv * E;
+      dst = v_cache + ((size_t)slot * Hv + g) * E;
     }
   }
   const T* src = qkv + (size_t)t * ld + col;
@@ -211,8 +213,7 @@ __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __
   }
   const float r = normed ? 1.0f / sqrtf(wave_sum(ss) / (float)size + unit_eps) : 1.0f;
   __syncthreads();
-  for (int c = 0; c < copies; ++c)
-    for (int i = threadIdx.x; i < size; i += blockDim.x) dst[(size_t)c * copy_stride + i] = from_f32<T>(staged[i] * r);
+  for (int i = threadIdx.x; i < size; i += blockDim.x) dst[i] = from_f32<T>(staged[i] * r);
 }
 
 extern "C" int nhv_rotary_split_write(const void* qkv, const void* bias, const void* qk_freqs, int rot, const void* v_freqs,

@@ -1556,10 +1556,12 @@ def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: t
     step's slots and returns q as [tokens, heads, head_dim]. Angles are taken in float from the position: no table.
     ``interleaved``: the pairs are (2i, 2i + 1). ``unit_eps``: after the rotation every query and key head is divided
     by its root mean square (this eps under the root), in float. ``values_from_keys``: the projection holds no value
-    columns; value head g is key head g as projected (not turned, not normed). ``maps`` n > 1: ``num_heads`` and
-    ``num_kv_heads`` count n maps per head, which lie in the projection as [head][map] and are returned and stored as
-    [map][head]; the projection holds num_kv_heads / n value heads, each stored once for every map (the value cache
-    has ``num_kv_heads`` heads)."""
+    columns; value head g is key head g as projected (not turned, not normed). ``maps`` n > 1: every query and key head
+    holds n maps of ``head_dim`` entries, each turned (and normed) on its own; ``num_heads`` and ``num_kv_heads`` count
+    maps. A key head's n maps are stored side by side as one key of n ``head_dim`` entries (the caches have
+    num_kv_heads / n heads, and the projection as many value heads); every query map is returned as a head of its own,
+    [tokens, num_heads, n head_dim], with zeros in the other maps' places, so that its product with a stored key is the
+    product with its own map."""
     T = qkv.shape[0]
     _need(maps >= 1 and num_heads % maps == 0 and num_kv_heads % maps == 0,
           lambda: f"rotary_split_write: {maps} maps with {num_heads} and {num_kv_heads} heads")
@@ -1589,16 +1591,16 @@ def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: t
     _dense(positions, "rotary_split_write: positions", (T,), torch.int32)
     if with_kv:
         _dense(slot_mapping, "rotary_split_write: slot_mapping", (T,), torch.int32)
-        _need(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (num_kv_heads, head_dim),
-              lambda: f"rotary_split_write: key cache {tuple(k_cache.shape)} does not fit {num_kv_heads} heads of {head_dim}")
-        _need(v_cache.dim() == 4 and tuple(v_cache.shape[2:]) == (num_kv_heads, value_dim),
-              lambda: f"rotary_split_write: value cache {tuple(v_cache.shape)} does not fit {num_kv_heads} heads of {value_dim}")
+        _need(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (num_kv_heads // maps, maps * head_dim),
+              lambda: f"rotary_split_write: key cache {tuple(k_cache.shape)} does not fit {num_kv_heads // maps} heads of {maps * head_dim}")
+        _need(v_cache.dim() == 4 and tuple(v_cache.shape[2:]) == (num_kv_heads // maps, value_dim),
+              lambda: f"rotary_split_write: value cache {tuple(v_cache.shape)} does not fit {num_kv_heads // maps} heads of {value_dim}")
         _dense(k_cache, "rotary_split_write: k_cache", dtype=qkv.dtype)
         _dense(v_cache, "rotary_split_write: v_cache", dtype=qkv.dtype)
         if v_freqs is not None:
             _need(value_dim % 2 == 0, "rotary_split_write: value heads of odd size cannot be turned")
             _float32(v_freqs, "rotary_split_write: value frequencies", (value_dim // 2,))
-    q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    q_out = torch.empty((T, num_heads, maps * head_dim), dtype=qkv.dtype, device=qkv.device)
     if T:
         backend().rotary_split_write(qkv, bias, qk_freqs, rot, v_freqs if with_kv else None, positions,
                                      slot_mapping if with_kv else None, q_out, k_cache if with_kv else None,
@@ -1608,7 +1610,8 @@ def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: t
 
 
 def differential_combine(a: torch.Tensor, lam: torch.Tensor, eps: float, post: float, gate: tuple | None = None) -> torch.Tensor:
-    """a [tokens, 2 heads, size] holds two softmax maps per head over the same values, map 1 of all heads first. Returns
+    """a [tokens, 2 heads, size] holds two softmax maps per head over the same values, per head its map 1, then its map
+    2. Returns
     [tokens, heads, size]: o = a1 - lam a2, divided by sqrt(mean(o^2) + eps) over the head's entries, times ``post``
     and, with ``gate`` = (rows [tokens, columns] of a's element type, first column), times sigmoid(rows[t, column + h]).
     ``lam``: one float32 number on the device."""

@@ -201,9 +201,10 @@ class DifferentialAttention(Part):
     with ``head_gate``, times sigmoid(w_h . x), x the mixer's input. Mask (``chunk`` or ``window``), grouping of heads,
     scale and rotation (``position``: a ``rotary_frequencies`` encoding; ``rotation`` "halves" or "interleaved") are
     those of ``RotaryAttention``; ``bias``: q, k, v and the output projection have biases.
-    To the cache and the attention kernels a map is a head: the step's queries go out as 2 ``num_heads`` heads, map 1
-    of all heads first, the keys as 2 ``num_kv_heads`` heads in the same order, so that the ordinary grouping of heads
-    pairs every map with its own keys; the values are stored once for every map."""
+    To the cache and the attention kernels a key head's two maps are one key of 2 ``head_dim`` entries, stored side by
+    side as projected, and a query map is a head of its own, 2 ``num_heads`` in all, of 2 ``head_dim`` entries with zeros
+    in the other map's place: its product with the stored key is the product with its own map. So keys and values
+    are stored once, in the sizes the projections give them, and the ordinary grouping of heads holds."""
 
     MAPS = 2
 
@@ -247,8 +248,9 @@ class DifferentialAttention(Part):
         self.lam = lam.to(torch.float32).reshape(1).contiguous()
 
     def cache_need(self):
-        return PagedKVNeed(self.MAPS * self.num_kv_heads, self.head_dim, self.window,
-                           None if self.value_dim == self.head_dim else self.value_dim, self.chunk)
+        key_dim = self.MAPS * self.head_dim
+        return PagedKVNeed(self.num_kv_heads, key_dim, self.window, None if self.value_dim == key_dim else self.value_dim,
+                           self.chunk)
 
     def forward(self, x, step, cache: CacheView):
         if not cache.writes:

@@ -271,7 +271,7 @@ class EmulatedBackend:
             x = (x + bias.float()).to(dt).float()
 
         def prepared(t):
-            """[T, heads, D] as projected -> turned, made unit vectors, the maps of all heads gathered map by map"""
+            """[T, heads, D] as projected -> turned, made unit vectors"""
             if rot and interleaved:
                 ang = positions.float()[:, None] * qk_freqs[None, :]
                 cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
@@ -282,29 +282,33 @@ class EmulatedBackend:
                 t = self._turned(t, positions, qk_freqs)
             if unit_eps is not None:
                 t = t / torch.sqrt((t * t).mean(-1, keepdim=True) + unit_eps)
-            if maps > 1:
-                t = t.reshape(T, t.shape[1] // maps, maps, D).transpose(1, 2).reshape(T, -1, D)
             return t
 
-        q_out.copy_(prepared(x[:, :Hq * D].reshape(T, Hq, D)).to(dt))
+        q = prepared(x[:, :Hq * D].reshape(T, Hq, D))
+        if maps > 1:                 # every map a head of its own, with zeros in the other maps' places
+            wide = torch.zeros(T, Hq, maps, D)
+            for s in range(Hq):
+                wide[:, s, s % maps] = q[:, s]
+            q = wide.reshape(T, Hq, maps * D)
+        q_out.copy_(q.to(dt))
         if with_kv:
             raw_k = x[:, Hq * D:(Hq + Hkv) * D].reshape(T, Hkv, D)
-            k = prepared(raw_k)
+            k = prepared(raw_k).reshape(T, Hkv // maps, maps * D)
             if values_from_keys:
                 v = raw_k
             else:
-                v = x[:, (Hq + Hkv) * D:].reshape(T, Hkv // maps, E).repeat(1, maps, 1)
+                v = x[:, (Hq + Hkv) * D:].reshape(T, Hkv // maps, E)
             if v_freqs is not None:
                 v = self._turned(v, positions, v_freqs)
             ok = slot_mapping >= 0
             slots = slot_mapping[ok].long()
-            k_cache.view(-1, Hkv, D)[slots] = k[ok].to(dt)
-            v_cache.view(-1, Hkv, E)[slots] = v[ok].to(dt)
+            k_cache.view(-1, Hkv // maps, maps * D)[slots] = k[ok].to(dt)
+            v_cache.view(-1, Hkv // maps, E)[slots] = v[ok].to(dt)
 
     def differential_combine(self, a, lam, out, eps, post, gate=None):
         T, H, E = out.shape
-        a = a.float()
-        o = a[:, :H] - lam.float() * a[:, H:]
+        a = a.float().reshape(T, H, 2, E)
+        o = a[:, :, 0] - lam.float() * a[:, :, 1]
         o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * post
         if gate is not None:
             o = o * torch.sigmoid(gate[0][:, gate[1]:gate[1] + H].float())[:, :, None]

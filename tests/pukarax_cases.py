@@ -72,7 +72,7 @@ CONFIG_B = model(50, 36, 1e-3, 1.0, 2.0, [
 # head sizes that the kernels on the matrix cores take (and one that they do not), a loop over all layers
 CONFIG_C = model(90, 64, 1e-6, 8.0, 0.25, [
     _with(keys_as_values(4, 2, 16, 11, 8, 10000.0, 8.0, 0.25), moe(6, 3, 16, 24)),
-    _with(two_maps(2, 2, 16, 16, 13, 16, 500000.0, 0.25, 0.5), dense(40)),
+    _with(two_maps(2, 2, 16, 32, 13, 16, 500000.0, 0.25, 0.5), dense(40)),
     _with(two_maps(4, 1, 32, 16, 20, 8, 300.0, 0.2, 0.45), moe(8, 2, 8, 8)),
 ], loop=(0, 3, 2))
 # recorded steps: a loop at the start
@@ -83,7 +83,7 @@ CONFIG_R = model(40, 32, 1e-5, 2.0, 1.0, [
 # the same kinds of sizes with chunks longer than a page of 64 tokens, one of them no multiple of it
 CONFIG_S = model(120, 64, 1e-6, 4.0, 0.5, [
     _with(keys_as_values(4, 2, 32, 150, 32, 50000.0, 8.0, 0.18), moe(6, 2, 16, 32)),
-    _with(two_maps(2, 1, 32, 32, 96, 32, 500000.0, 0.18, 0.5), dense(48)),
+    _with(two_maps(2, 1, 32, 64, 96, 32, 500000.0, 0.18, 0.5), dense(48)),
     _with(two_maps(2, 2, 16, 48, 128, 16, 500000.0, 0.25, 0.4), moe(4, 2, 16)),
 ], loop=(0, 2, 2))
 # the sizes of a real model's layers in small number: heads of 128 and 64, a width of 1,024
@@ -179,7 +179,7 @@ def random_config(seed: int) -> dict:
         rot = r.choice([0, 2, dim // 2 // 2 * 2, dim])
         scale = r.choice([0.5, 1.0, 2.0]) * dim ** -0.5
         if r.random() < 0.5:
-            vdim = dim if r.random() < 0.5 else r.choice([4, 12, 16, 24])
+            vdim = 2 * dim if r.random() < 0.5 else r.choice([4, 12, 16, 24, dim])
             entry = two_maps(heads, kv, dim, vdim, chunk, rot, r.choice([10.0, 1000.0, 500000.0]), scale, r.choice([0.2, 0.5, 0.8]))
         else:
             entry = keys_as_values(heads, kv, dim, chunk, rot, r.choice([10.0, 1000.0, 50000.0]), r.choice([None, 2.0, 8.0]), scale)

@@ -426,7 +426,7 @@ def _compare(got, want, dtype, what):
             allowed = tol + 10.0 * getattr(want, "moved", {}).get(rid, torch.zeros_like(errors))
             assert bool((errors <= allowed).all()), (what, rid, (errors > allowed).nonzero().flatten().tolist()[:4], float(errors.max()))
         return
-    errors = torch.cat([(got[rid].float() - want[rid].float()).abs().max(dim=-1).values for rid in want])
+    errors = torch.cat([(got[rid].float() - want[rid].float()).pow(2).mean(dim=-1).sqrt() for rid in want])    # (over the vocabulary)
     assert bool(torch.isfinite(errors).all()), what
     assert float((errors > tol).float().mean()) <= 0.1 and float(errors.max()) <= 20 * tol, \
         (what, float((errors > tol).float().mean()), float(errors.max()) / tol)

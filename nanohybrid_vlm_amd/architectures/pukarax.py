@@ -268,12 +268,12 @@ def _shape(layers: int, width: int, ff: int, vocab: int, heads: int, kv_heads: i
         if differential_every and i % differential_every == differential_every - 1:
             half = dim // 2
             entry = {"type": "attention",
-                     "mixer": {"diff": 0.5, "dim": half, "heads": heads, "kv_heads": kv_heads, "mask": {"size": chunk},
-                               "rot": {"base": 500000.0, "dims": half}, "scale": half ** -0.5, "vdim": dim}}
+                     "mixer": {"diff": 0.4, "dim": half, "heads": heads, "kv_heads": kv_heads, "mask": {"size": chunk},
+                               "rot": {"base": 100000.0, "dims": half}, "scale": half ** -0.5, "vdim": dim}}
         else:
             entry = {"type": "attention_2",
                      "mixer": {"dim": dim, "heads": heads, "kv_heads": kv_heads, "mask": {"size": chunk},
-                               "rot": {"base": 50000.0, "dims": dim, "scaling": {"factor": 8.0}}, "scale": dim ** -0.5,
+                               "rot": {"base": 10000.0, "dims": dim, "scaling": {"factor": 4.0}}, "scale": dim ** -0.5,
                                "vdim": dim}}
         if experts and i % 2:
             entry["mlp"] = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top},

@@ -70,26 +70,26 @@ CONFIG_B = model(50, 36, 1e-3, 1.0, 2.0, [
     _with(two_maps(3, 3, 2, 5, 1, 2, 7.0, 1.0, 0.1), None),
 ])
 # head sizes that the kernels on the matrix cores take (and one that they do not), a loop over all layers
-CONFIG_C = model(90, 64, 1e-6, 8.0, 0.25, [
-    _with(keys_as_values(4, 2, 16, 11, 8, 10000.0, 8.0, 0.25), moe(6, 3, 16, 24)),
-    _with(two_maps(2, 2, 16, 32, 13, 16, 500000.0, 0.25, 0.5), dense(40)),
+CONFIG_C = model(90, 64, 2e-6, 8.0, 0.2, [
+    _with(keys_as_values(4, 2, 16, 11, 8, 10000.0, 16.0, 0.25), moe(6, 3, 16, 24)),
+    _with(two_maps(2, 2, 16, 32, 13, 16, 300000.0, 0.25, 0.35), dense(40)),
     _with(two_maps(4, 1, 32, 16, 20, 8, 300.0, 0.2, 0.45), moe(8, 2, 8, 8)),
 ], loop=(0, 3, 2))
 # recorded steps: a loop at the start
 CONFIG_R = model(40, 32, 1e-5, 2.0, 1.0, [
-    _with(two_maps(2, 1, 16, 16, 8, 8, 100.0, 0.3, 0.5), moe(4, 2, 8, 8)),
+    _with(two_maps(2, 1, 16, 16, 8, 8, 100.0, 0.3, 0.45), moe(4, 2, 8, 8)),
     _with(keys_as_values(2, 1, 16, 12, 16, 1000.0, 2.0, 0.3), dense(16)),
 ], loop=(0, 1, 2))
 # the same kinds of sizes with chunks longer than a page of 64 tokens, one of them no multiple of it
 CONFIG_S = model(120, 64, 1e-6, 4.0, 0.5, [
-    _with(keys_as_values(4, 2, 32, 150, 32, 50000.0, 8.0, 0.18), moe(6, 2, 16, 32)),
-    _with(two_maps(2, 1, 32, 64, 96, 32, 500000.0, 0.18, 0.5), dense(48)),
-    _with(two_maps(2, 2, 16, 48, 128, 16, 500000.0, 0.25, 0.4), moe(4, 2, 16)),
+    _with(keys_as_values(4, 2, 32, 150, 32, 20000.0, 4.0, 0.18), moe(6, 2, 16, 32)),
+    _with(two_maps(2, 1, 32, 64, 80, 32, 300000.0, 0.18, 0.55), dense(48)),
+    _with(two_maps(2, 2, 16, 48, 128, 16, 300000.0, 0.25, 0.4), moe(4, 2, 16)),
 ], loop=(0, 2, 2))
 # the sizes of a real model's layers in small number: heads of 128 and 64, a width of 1,024
 CONFIG_W = model(500, 1024, 1e-6, 32.0, 0.1, [
-    _with(keys_as_values(8, 2, 128, 256, 128, 50000.0, 8.0, 0.09), moe(8, 2, 256, 512)),
-    _with(two_maps(8, 4, 64, 128, 192, 64, 500000.0, 0.125, 0.5), dense(2048)),
+    _with(keys_as_values(8, 2, 128, 256, 128, 20000.0, 4.0, 0.09), moe(8, 2, 256, 512)),
+    _with(two_maps(8, 4, 64, 128, 192, 64, 300000.0, 0.125, 0.6), dense(2048)),
 ])
 
 CASES = {"A": (CONFIG_A, 31), "B": (CONFIG_B, 42), "C": (CONFIG_C, 33), "R": (CONFIG_R, 34), "S": (CONFIG_S, 35)}
@@ -180,9 +180,9 @@ def random_config(seed: int) -> dict:
         scale = r.choice([0.5, 1.0, 2.0]) * dim ** -0.5
         if r.random() < 0.5:
             vdim = 2 * dim if r.random() < 0.5 else r.choice([4, 12, 16, 24, dim])
-            entry = two_maps(heads, kv, dim, vdim, chunk, rot, r.choice([10.0, 1000.0, 500000.0]), scale, r.choice([0.2, 0.5, 0.8]))
+            entry = two_maps(heads, kv, dim, vdim, chunk, rot, r.choice([10.0, 1000.0, 300000.0]), scale, r.choice([0.2, 0.4, 0.8]))
         else:
-            entry = keys_as_values(heads, kv, dim, chunk, rot, r.choice([10.0, 1000.0, 50000.0]), r.choice([None, 2.0, 8.0]), scale)
+            entry = keys_as_values(heads, kv, dim, chunk, rot, r.choice([10.0, 1000.0, 20000.0]), r.choice([None, 2.0, 16.0]), scale)
         kind = r.choice(["none", "dense", "moe", "moe"])
         if kind == "dense":
             entry["mlp"] = dense(r.choice([16, 24, 50]))
@@ -197,4 +197,4 @@ def random_config(seed: int) -> dict:
         start = r.randint(0, len(layers) - 1)
         loop = (start, r.randint(start, len(layers)), r.randint(1, 3))
     return model(r.choice([33, 64, 90, 131]), width, r.choice([1e-6, 1e-5, 1e-3]), r.choice([1.0, 4.0, 10.0]),
-                 r.choice([0.25, 1.0, 2.0]), layers, loop)
+                 r.choice([0.3, 1.0, 2.0]), layers, loop)

@@ -507,7 +507,7 @@ def test_configurations_drawn_at_random(where, kernels, seed, tmp_path):
 
 @pytest.mark.parametrize("where", ON_GPU)
 def test_pages_of_64_and_chunks_longer_than_a_page(folders, where, kernels):
-    """Pages of 64 tokens (whole tiles of the prompt kernel lie in one page) under chunks of 96, 128 and 150 positions,
+    """Pages of 64 tokens (whole tiles of the prompt kernel lie in one page) under chunks of 80, 128 and 150 positions,
     requests of up to 400 tokens in portions that end anywhere, beside decoded tokens, on few pages."""
     device, dtype = where
     requests = _requests("S", [400, 130, 70, 257])

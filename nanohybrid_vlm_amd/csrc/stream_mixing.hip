@@ -162,7 +162,7 @@ __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __
                                           T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq,
                                           int Hkv, int Hv, int D, int E, int heads, int ld, int interleaved, int unit,
                                           float unit_eps, int v_from_k, int maps) {
-  extern __shared__ float staged[];            // max(D, E) floats: the head after bias and rotation
+  extern __shared__ float staged[];            // D floats where heads are normed: the head after bias and rotation
   const int t = blockIdx.x / heads, head = blockIdx.x % heads;
   const float p = (float)positions[t];
   int col, size, half;
@@ -194,6 +194,22 @@ __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __
   const T* bs = bias ? bias + col : nullptr;
   // the bias joins a projection that was rounded to the rows' type, and the sum is rounded again (the product's own result)
   auto value = [&](int i) { return bs ? to_f32(from_f32<T>(to_f32(src[i]) + to_f32(bs[i]))) : to_f32(src[i]); };
+  if (!normed) {                               // nothing of the head depends on all of it: every entry goes out at once
+    for (int i = threadIdx.x; i < size - half; i += blockDim.x) {
+      if (i < half) {
+        const int a = pairs_adjacent ? 2 * i : i, b = pairs_adjacent ? 2 * i + 1 : i + half;
+        const float u = value(a), v = value(b);
+        float sn, cs;
+        sincosf(p * freqs[i], &sn, &cs);
+        dst[a] = from_f32<T>(u * cs - v * sn);
+        dst[b] = from_f32<T>(v * cs + u * sn);
+      } else {
+        dst[i + half] = from_f32<T>(value(i + half));
+      }
+    }
+    return;
+  }
+  // the unit norm follows the rotation: the turned head waits in LDS as floats for its sum of squares
   float ss = 0.f;
   for (int i = threadIdx.x; i < size - half; i += blockDim.x) {
     if (i < half) {
@@ -211,7 +227,7 @@ __global__ void rotary_split_write_kernel(const T* __restrict__ qkv, const T* __
       ss = fmaf(x, x, ss);
     }
   }
-  const float r = normed ? 1.0f / sqrtf(wave_sum(ss) / (float)size + unit_eps) : 1.0f;
+  const float r = 1.0f / sqrtf(wave_sum(ss) / (float)size + unit_eps);
   __syncthreads();
   for (int i = threadIdx.x; i < size; i += blockDim.x) dst[i] = from_f32<T>(staged[i] * r);
 }
@@ -234,8 +250,8 @@ extern "C" int nhv_rotary_split_write(const void* qkv, const void* bias, const v
   const int heads = with_kv ? Hq + Hkv + Hv : Hq;
   const int ld = (with_kv ? Hq * D + Hkv * D + (v_from_k ? 0 : Hv * E) : Hq * D) + more_columns;   // (columns that belong to another reader)
   NHV_REQUIRE((long long)T * heads < (1ll << 31), "rotary_split_write: too many tokens");
-  const size_t lds = (size_t)(D > E ? D : E) * sizeof(float);
-  NHV_REQUIRE(lds <= 64 * 1024, "rotary_split_write: heads of %d and %d entries are beyond this kernel", D, E);
+  const size_t lds = unit ? (size_t)D * sizeof(float) : 0;
+  NHV_REQUIRE(lds <= 64 * 1024, "rotary_split_write: heads of %d entries are beyond this kernel's unit norm", D);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(TT)                                                                                                   \
   hipLaunchKernelGGL(rotary_split_write_kernel<TT>, dim3((unsigned)((size_t)T * heads)), dim3(NHV_WAVE), lds, s,     \

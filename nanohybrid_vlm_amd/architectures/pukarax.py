@@ -17,10 +17,10 @@ config.json: {"architecture": "Pukarax", "vocab", "width", "norm": {"eps"}, "emb
   heads over ``kv_heads`` key/value heads; ``scale`` multiplies the scores.
 * ``mlp.kind`` "dense": down(silu(gate x) * (up x)) of inner size ``ff``. "moe": ``router.experts`` such feed-forwards
   of inner size ``expert.ff`` without biases, of which a token uses the ``router.top`` with the largest router logit
-  (router weight and bias); their weights are the softmax over the chosen logits and weigh the experts' outputs; with
-  ``shared`` ({"ff"}) one more such feed-forward runs for every token and is added.
-* ``loop``: the layers start .. stop - 1 run ``times`` times in a row as a group, with the same weights and a cache
-  of its own for every run.
+  (router weight and bias); the experts' outputs are summed with softmax(chosen logits) as their weights; ``shared``
+  ({"ff"}) names one more such feed-forward that all tokens use, added to that sum.
+* ``loop``: the group of layers start .. stop - 1 is run ``times`` times over before the layers after it, on one set
+  of weights, every run with a cache of its own.
 
 The embedding's rows are multiplied by ``embedding.scale``; the head is the embedding table (unscaled) and the logits
 are multiplied by ``logit_scale``.

@@ -7,7 +7,7 @@ The design in this file's notation (x the stream, h a sublayer's input, p a posi
 
 * x0 = E[token] * s_e.
 * a layer: x += N1b(mixer(N1(x))); x += N2b(ff(N2(x))) with N(v) = v / sqrt(mean(v^2) + eps) * w; layers
-  ``loop.start`` to ``loop.stop - 1`` run ``loop.times`` times in a row as a group, with the same weights.
+  ``loop.start`` to ``loop.stop - 1`` are a group that is run ``loop.times`` times over, on one set of weights.
 * mixer "attention" (two softmax maps per head, their difference): q and k hold per head [map 1 | map 2]; both
   maps are turned over their first ``rot.dims`` entries, pairs (2i, 2i + 1), angle p * base^(-2i / dims); the maps
   read the same values; lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff; o = a1 - lambda a2, divided by its root mean
@@ -16,8 +16,8 @@ The design in this file's notation (x the stream, h a sublayer's input, p a posi
   angle p * base^(-2i / dims) / factor, then divided by their root mean square per head; the concatenated heads are
   multiplied entry by entry with sigmoid(G h); no biases.
 * both: scores q . k * scale; position i reads j <= i with floor(i / size) = floor(j / size); grouped key/value heads.
-* feed-forward "dense": D(silu(G h) * (U h)). "moe": z = R h + b; the ``top`` largest z are chosen, their weights are
-  the softmax over the chosen z; the weighted sum of the chosen experts' outputs plus a shared expert.
+* feed-forward "dense": D(silu(G h) * (U h)). "moe": z = R h + b; the ``top`` largest z win (the lower number among
+  equals), softmax(winners' z) weighs the winners' outputs, and a shared expert's output is added.
 * logits = E N_f(x) * s_l.
 """
 from __future__ import annotations
